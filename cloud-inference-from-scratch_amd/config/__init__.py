@@ -1,5 +1,6 @@
 from .engine_config import EngineConfig, build_engine_config, canonical_dtype
 from .givizen import GivizenConfig
+from .nokipel import NokipelConfig
 from .polosun import PolosunConfig
 from .qwen2 import Qwen2Config
 from .registry import (
@@ -16,9 +17,10 @@ from .specs import ConfigError, LayerCall, LayerSpec, ModelSpec, PartSpec
 register_architecture("Qwen2ForCausalLM", Qwen2Config, model_type="qwen2")
 register_architecture("Polosun", PolosunConfig)
 register_architecture("Givizen", GivizenConfig)
+register_architecture("Nokipel", NokipelConfig)
 
 __all__ = [
     "ARCHITECTURES", "Architecture", "ConfigError", "EngineConfig", "GivizenConfig", "LayerCall", "LayerSpec",
-    "ModelSpec", "PartSpec", "PolosunConfig", "Qwen2Config", "architecture_of", "build_engine_config",
+    "ModelSpec", "NokipelConfig", "PartSpec", "PolosunConfig", "Qwen2Config", "architecture_of", "build_engine_config",
     "canonical_dtype", "config_from_dict", "load_config", "register_architecture",
 ]

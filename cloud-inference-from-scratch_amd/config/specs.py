@@ -69,11 +69,14 @@ class LayerCall:
                same unit, then the later one reads what the earlier one wrote.
     ``writes`` whether this call appends its own keys/values (or state) to the
                unit before reading it.
+    ``adds_embedding`` the embedding's rows (scaled, as they entered the stream) join the
+               stream once more right in front of this call.
     """
 
     layer: int
     cache: int
     writes: bool = True
+    adds_embedding: bool = False
 
 
 @dataclass(frozen=True)

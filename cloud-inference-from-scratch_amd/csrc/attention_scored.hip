@@ -5,6 +5,7 @@
 //   s_ij <- cap * tanh(s_ij / cap)                       cap > 0
 //   s_ij <- s_ij - slope[head] * (i - j)                 slopes given (a bias on the distance itself)
 //   j is seen by i when 0 <= i - j < window              window > 0 (else every j <= i)
+//   ... or when j <= i and floor(i / chunk) = floor(j / chunk)   chunk > 0: chunks counted from position 0
 //   p_ij = exp(s_ij) / (sum_j exp(s_ij) + exp(sink[head]))   sinks given: one more term in the denominator, which
 //                                                        has no key and no value, no scale and no bias
 //   o_i  = sum_j p_ij v_j,  o_i <- o_i * sigmoid(gate[i, head])   gate given
@@ -16,6 +17,8 @@
 // `cie_heads_prepare` is what stands between the projection and this attention: a per-head RMS norm of queries
 // and keys (with a weight, without one, or none), the queries' factor that grows with the position,
 //   q <- q * (1 + coef * ln(floor((p + 1) / every) + 1)),
+// then a rotation of the first `rot` numbers of every query and key head by the position (pairs of neighbours or of
+// the two halves; cos and sin from float32 tables [positions, rot / 2]),
 // queries laid out [tokens, heads, D] (zero-padded from the projection's head size up to D) and keys and values
 // written to the cache (padded likewise).  Statistics, the logarithm and the scaling are float32.
 #include "attention_args.h"
@@ -35,7 +38,8 @@ heads_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int
                      const int* __restrict__ seq_of_token, const int* __restrict__ seq_slot,
                      const int* __restrict__ block_table, int table_width, T* __restrict__ q_out,
                      T* __restrict__ k_pool, T* __restrict__ v_pool, int tokens, int q_heads, int kv_heads,
-                     int dim, int vdim, int D, int DV, int page_shift, int write_kv) {
+                     int dim, int vdim, int D, int DV, int page_shift, int write_kv,
+                     const float* __restrict__ cos_table, const float* __restrict__ sin_table, int rot, int neighbours) {
     const int lane = threadIdx.x % kWave;
     const int slots = q_heads + 2 * kv_heads;
     const long unit = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
@@ -77,11 +81,25 @@ heads_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int
         after = 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every) + 1.0f);
     T* dst = is_q ? q_out + (static_cast<size_t>(token) * q_heads + head) * D
                   : k_pool + (((page * kv_heads + head) << page_shift) + (pos & (page_size - 1))) * D;
+    const int half = rot / 2;
+    const float* cos_row = rot > 0 ? cos_table + static_cast<size_t>(pos) * half : nullptr;
+    const float* sin_row = rot > 0 ? sin_table + static_cast<size_t>(pos) * half : nullptr;
     for (int d = lane; d < D; d += kWave) {
         float x = 0.f;
         if (d < dim) {
             x = to_float(src[d]) * factor;
             if (norm_mode == 2) x *= weight[d];
+            if (d < rot) {
+                // the pair (u, v) of the angle's index i turns to (u cos - v sin, v cos + u sin): neighbours
+                // (2i, 2i + 1) or the halves (i, i + rot / 2)
+                const int i = neighbours ? d >> 1 : (d < half ? d : d - half);
+                const bool is_u = neighbours ? !(d & 1) : d < half;
+                const int mate = neighbours ? d ^ 1 : (is_u ? d + half : d - half);
+                float y = to_float(src[mate]) * factor;
+                if (norm_mode == 2) y *= weight[mate];
+                const float c = cos_row[i], sn = sin_row[i];
+                x = is_u ? x * c - y * sn : x * c + y * sn;
+            }
             x *= after;
         }
         dst[d] = from_float<T>(x);
@@ -120,7 +138,14 @@ struct ScoreShape {
     const float* slopes;  // [q_heads] or null
     const float* sinks;   // [q_heads] or null
     int window;           // <= 0: all keys
+    int chunk;            // > 0: i sees j <= i only inside its own chunk, floor(i / chunk) == floor(j / chunk)
 };
+
+// The first key that the query at position `pos` sees.
+__device__ __forceinline__ int first_seen(int pos, int window, int chunk) {
+    if (chunk > 0) return pos < 0 ? 0 : pos - pos % chunk;
+    return window > 0 ? max(0, pos + 1 - window) : 0;
+}
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -143,7 +168,7 @@ scored_attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ k
     const int kv_head = head / (q_heads / kv_heads);
     const int pos = positions[token];
     const int len = pos + 1;
-    const int lo = (shape.window > 0 && len > shape.window) ? len - shape.window : 0;
+    const int lo = first_seen(pos, shape.window, shape.chunk);
     const int* table = block_table + static_cast<size_t>(seq_slot[seq_of_token[token]]) * table_width;
     const float slope = shape.slopes ? shape.slopes[head] : 0.f;
 
@@ -305,7 +330,8 @@ __global__ void __launch_bounds__(64 * kScoredWaves, RT <= 2 ? 2 : 1) scored_att
     const int window = a.shape.window;
 
     const int hi = start + q0 + n_tok;
-    const int lo = (window > 0) ? max(0, start + q0 + 1 - window) : 0;
+    const int chunk = a.shape.chunk;
+    const int lo = first_seen(start + q0, window, chunk);
     int range_begin = lo & ~(kKeysPerBlock - 1);
     int range_end = hi;
     const int split = blockIdx.z;
@@ -314,7 +340,7 @@ __global__ void __launch_bounds__(64 * kScoredWaves, RT <= 2 ? 2 : 1) scored_att
         range_end = min(hi, range_begin + a.keys_per_split);
     }
     const int first_pos = start + q0;            // position of the tile's first token (its window reaches back furthest)
-    const int last_lo = (window > 0) ? start + q0 + n_tok - window : 0;  // the first key the tile's last token sees
+    const int last_lo = first_seen(start + q0 + n_tok - 1, window, chunk);  // the first key the tile's last token sees
 
     if (a.n_splits > 1 && range_begin >= range_end) {  // a share without keys: its statistics say so, its sums are never read
         float* pml = a.part_ml + ((static_cast<size_t>(tile) * a.kv_heads + kv_head) * a.n_splits + split) * ROWS * 2;
@@ -390,7 +416,7 @@ __global__ void __launch_bounds__(64 * kScoredWaves, RT <= 2 ? 2 : 1) scored_att
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             const int pos = row_pos[rt];
-            const int row_lo = (window > 0) ? pos + 1 - window : 0;
+            const int row_lo = first_seen(pos, window, chunk);
             float block_max = -INFINITY;
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt) {
@@ -621,7 +647,9 @@ CIE_API int cie_heads_prepare(void* stream, int dtype, const void* proj, int pro
                               float temp_coef, int temp_every, const int* positions, const int* seq_of_token,
                               const int* seq_slot, const int* block_table, int table_width, void* q_out,
                               void* k_pool, void* v_pool, int tokens, int q_heads, int kv_heads, int dim, int vdim,
-                              int D, int DV, int page_size, int write_kv) {
+                              int D, int DV, int page_size, int write_kv, const float* cos_table,
+                              const float* sin_table, int rot, int neighbours) {
+    if (rot < 0 || rot % 2 || rot > dim || (rot > 0 && (!cos_table || !sin_table))) return CIE_BAD_ARGUMENT;
     if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || D < dim || DV < vdim ||
         page_size <= 0 || (page_size & (page_size - 1)) || table_width <= 0 || norm_mode < 0 || norm_mode > 2 ||
         (norm_mode == 2 && (!q_weight || !k_weight)) || (norm_mode != 0 && !(eps > 0.f)) || temp_every < 0 ||
@@ -639,13 +667,13 @@ CIE_API int cie_heads_prepare(void* stream, int dtype, const void* proj, int pro
             static_cast<const float*>(proj), proj_stride, q_off, k_off, v_off, q_weight, k_weight, norm_mode, eps,
             temp_coef, temp_every, positions, seq_of_token, seq_slot, block_table, table_width,
             static_cast<float*>(q_out), static_cast<float*>(k_pool), static_cast<float*>(v_pool), tokens, q_heads,
-            kv_heads, dim, vdim, D, DV, page_shift, write_kv);
+            kv_heads, dim, vdim, D, DV, page_shift, write_kv, cos_table, sin_table, rot, neighbours);
     else if (dtype == CIE_BF16)
         heads_prepare_kernel<bf16_t><<<static_cast<unsigned>(blocks), 256, 0, s>>>(
             static_cast<const bf16_t*>(proj), proj_stride, q_off, k_off, v_off, q_weight, k_weight, norm_mode, eps,
             temp_coef, temp_every, positions, seq_of_token, seq_slot, block_table, table_width,
             static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_pool), static_cast<bf16_t*>(v_pool), tokens, q_heads,
-            kv_heads, dim, vdim, D, DV, page_shift, write_kv);
+            kv_heads, dim, vdim, D, DV, page_shift, write_kv, cos_table, sin_table, rot, neighbours);
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();
@@ -656,7 +684,7 @@ CIE_API int cie_scored_attention_generic(void* stream, int dtype, const void* q,
                                          const int* positions, const int* seq_of_token, const int* seq_slot,
                                          const void* gate, int gate_stride, void* out, int tokens, int q_heads,
                                          int kv_heads, int D, int DV, int page_size, int window, float scale,
-                                         float softcap, const float* slopes, const float* sinks) {
+                                         float softcap, const float* slopes, const float* sinks, int chunk) {
     if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || D <= 0 || D % 8 || DV <= 0 || DV % 8 ||
         D > kWave * kMaxSlices || DV > kWave * kMaxSlices || page_size <= 0 || table_width <= 0 || q_heads > 65535 ||
         (gate && gate_stride < q_heads))
@@ -665,7 +693,8 @@ CIE_API int cie_scored_attention_generic(void* stream, int dtype, const void* q,
     hipStream_t s = static_cast<hipStream_t>(stream);
     dim3 grid(tokens, q_heads);
     const size_t lds = (static_cast<size_t>(D) + 4 * DV) * sizeof(float);
-    const ScoreShape shape{scale, softcap, slopes, sinks, window};
+    if (chunk < 0 || (chunk > 0 && window > 0)) return CIE_BAD_ARGUMENT;
+    const ScoreShape shape{scale, softcap, slopes, sinks, window, chunk};
     if (dtype == CIE_F32)
         scored_attention_generic_kernel<float><<<grid, 256, lds, s>>>(
             static_cast<const float*>(q), static_cast<const float*>(k_pool), static_cast<const float*>(v_pool),
@@ -690,7 +719,8 @@ CIE_API int cie_scored_attention_mfma(void* stream, const void* q, const void* k
                                       int gate_stride, void* out, int q_heads, int kv_heads, int D, int DV,
                                       int page_size, int tokens_per_tile, int row_tiles, int window, float scale,
                                       float softcap, const float* slopes, const float* sinks, int n_splits,
-                                      int keys_per_split, float* part_o, float* part_ml) {
+                                      int keys_per_split, float* part_o, float* part_ml, int chunk) {
+    if (chunk < 0 || (chunk > 0 && window > 0)) return CIE_BAD_ARGUMENT;
     if (n_tiles < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || page_size < 4 ||
         (page_size & (page_size - 1)) || table_width <= 0 || tokens_per_tile < 1 || kv_heads > 65535 ||
         (tile_seq == nullptr) != (tile_q0 == nullptr) || (gate && gate_stride < q_heads))
@@ -725,7 +755,7 @@ CIE_API int cie_scored_attention_mfma(void* stream, const void* q, const void* k
     while ((1 << a.page_shift) < page_size) ++a.page_shift;
     a.tokens_per_tile = tokens_per_tile;
     a.n_tiles = n_tiles;
-    a.shape = ScoreShape{scale, softcap, slopes, sinks, window};
+    a.shape = ScoreShape{scale, softcap, slopes, sinks, window, chunk};
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (D == 64 && DV == 64) return launch_scored<64, 64>(s, a, row_tiles);
     if (D == 128 && DV == 128) return launch_scored<128, 128>(s, a, row_tiles);

@@ -207,3 +207,91 @@ CIE_API int cie_branch_norm_add(void* stream, int bdtype, int dtype, float* resi
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();
 }
+
+// ---------------------------------------------------------------------------------------------- norm in groups
+// The residual add of a layer that norms what its sublayers read, with everything a branch can still owe the stream,
+// and an RMS norm whose statistics run over equal consecutive parts of the row:
+//
+//   x = residual[row] + branch[row] * sigmoid(branch_gate[row])            (branch; the gate one logit per row)
+//                     + sum_p part_weight[row, p] * parts[row, p, :]       (float32 rows still to be summed, in order)
+//                     + plus[row]                                          (float32 rows, e.g. the embedding's again)
+//   y[g] = x[g] / sqrt(mean(x[g]^2) + eps) * weight[g]                     for each of the `groups` parts g of the row
+//
+// Every addend may be absent.  Sums, statistics and scaling are float32; the row is staged in LDS.  With `rows`
+// given only those rows are normed and the stream is not written back.  A wave takes the groups in turn, so the
+// statistics need no barrier per group.
+template <typename B, typename T>
+__global__ void group_norm_add_kernel(float* __restrict__ residual, const B* __restrict__ branch,
+                                      const float* __restrict__ branch_gate, const float* __restrict__ parts,
+                                      const float* __restrict__ part_weight, int n_parts,
+                                      const float* __restrict__ plus, const float* __restrict__ weight,
+                                      T* __restrict__ out, const int* __restrict__ rows, int hidden, int groups,
+                                      float eps, int write_residual) {
+    extern __shared__ float staged[];  // [hidden], then [groups]
+    float* inverse = staged + hidden;
+    const int out_row = blockIdx.x;
+    const size_t row = rows ? rows[out_row] : out_row;
+    float* res = residual + row * hidden;
+    const B* add = branch ? branch + row * hidden : nullptr;
+    const float open = (branch && branch_gate) ? 1.0f / (1.0f + expf(-branch_gate[row])) : 1.0f;
+    const float* extra = n_parts > 0 ? parts + row * n_parts * hidden : nullptr;
+    const float* extra_w = (n_parts > 0 && part_weight) ? part_weight + row * n_parts : nullptr;
+    const float* more = plus ? plus + row * hidden : nullptr;
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
+        float x = res[h];
+        if (add) x += to_float(add[h]) * open;
+        for (int p = 0; p < n_parts; ++p)
+            x += (extra_w ? extra_w[p] : 1.0f) * extra[static_cast<size_t>(p) * hidden + h];
+        if (more) x += more[h];
+        if (write_residual) res[h] = x;
+        staged[h] = x;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x % kWave;
+    const int waves = blockDim.x / kWave;
+    const int per = hidden / groups;
+    for (int g = threadIdx.x / kWave; g < groups; g += waves) {
+        float sum_sq = 0.f;
+        for (int h = lane; h < per; h += kWave) {
+            const float x = staged[g * per + h];
+            sum_sq += x * x;
+        }
+        sum_sq = wave_sum(sum_sq);
+        if (lane == 0) inverse[g] = 1.0f / sqrtf(sum_sq / static_cast<float>(per) + eps);
+    }
+    __syncthreads();
+    T* dst = out + static_cast<size_t>(out_row) * hidden;
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x)
+        dst[h] = from_float<T>((staged[h] * inverse[h / per]) * weight[h]);
+}
+
+// bdtype: storage type of `branch` (ignored without one); dtype: type of `out`.  `weight` float32 [hidden].
+CIE_API int cie_group_norm_add(void* stream, int bdtype, int dtype, float* residual, const void* branch,
+                               const float* branch_gate, const float* parts, const float* part_weight, int n_parts,
+                               const float* plus, const float* weight, void* out, const int* rows, int n_rows,
+                               int hidden, int groups, float eps) {
+    if (n_rows < 0 || hidden <= 0 || groups <= 0 || hidden % groups || !(eps > 0.f) || n_parts < 0 ||
+        (n_parts > 0 && !parts) || (static_cast<size_t>(hidden) + groups) * sizeof(float) > 64 * 1024 || !weight || !out)
+        return CIE_BAD_ARGUMENT;
+    if (n_rows == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int threads = n_rows <= 64 ? 1024 : 256;
+    const size_t lds = (static_cast<size_t>(hidden) + groups) * sizeof(float);
+    if (!parts) n_parts = 0;
+    const int write_residual = (rows == nullptr && (branch || n_parts > 0 || plus)) ? 1 : 0;
+    if (dtype == CIE_F32 && (bdtype == CIE_F32 || !branch))
+        group_norm_add_kernel<float, float><<<n_rows, threads, lds, s>>>(
+            residual, static_cast<const float*>(branch), branch_gate, parts, part_weight, n_parts, plus, weight,
+            static_cast<float*>(out), rows, hidden, groups, eps, write_residual);
+    else if (dtype == CIE_BF16 && (bdtype == CIE_BF16 || !branch))
+        group_norm_add_kernel<bf16_t, bf16_t><<<n_rows, threads, lds, s>>>(
+            residual, static_cast<const bf16_t*>(branch), branch_gate, parts, part_weight, n_parts, plus, weight,
+            static_cast<bf16_t*>(out), rows, hidden, groups, eps, write_residual);
+    else if (dtype == CIE_BF16 && bdtype == CIE_F32)
+        group_norm_add_kernel<float, bf16_t><<<n_rows, threads, lds, s>>>(
+            residual, static_cast<const float*>(branch), branch_gate, parts, part_weight, n_parts, plus, weight,
+            static_cast<bf16_t*>(out), rows, hidden, groups, eps, write_residual);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}

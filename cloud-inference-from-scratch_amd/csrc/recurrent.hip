@@ -20,6 +20,9 @@ namespace {
 
 __device__ __forceinline__ float sigmoidf(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+// what stands between a projection and the memory: 0 nothing, 1 silu
+__device__ __forceinline__ float activated(float z, int act) { return act == 1 ? z * sigmoidf(z) : z; }
+
 __device__ __forceinline__ float gelu_tanh(float z) {
     return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
@@ -42,7 +45,7 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 retention_turn_kernel(const T* __restrict__ proj, long ldp, int q_off, int k_off, const float* __restrict__ cos_table,
                       const float* __restrict__ sin_table, int rot, const int* __restrict__ positions,
-                      float* __restrict__ turned, int heads, int dim, int padded, float key_scale) {
+                      float* __restrict__ turned, int heads, int dim, int padded, float key_scale, int act) {
     const int token = blockIdx.x;
     const int half = rot / 2;
     const T* row = proj + static_cast<size_t>(token) * ldp;
@@ -54,17 +57,17 @@ retention_turn_kernel(const T* __restrict__ proj, long ldp, int q_off, int k_off
         if (d < dim) {
             const T* qh = row + q_off + head * dim;
             const T* kh = row + k_off + head * dim;
-            qv = to_float(qh[d]);
-            kv = to_float(kh[d]);
+            qv = activated(to_float(qh[d]), act);
+            kv = activated(to_float(kh[d]), act);
             if (d < rot) {
                 const int i = d < half ? d : d - half;
                 const float c = cos_table[at + i], s = sin_table[at + i];
                 if (d < half) {
-                    qv = qv * c - to_float(qh[d + half]) * s;
-                    kv = kv * c - to_float(kh[d + half]) * s;
+                    qv = qv * c - activated(to_float(qh[d + half]), act) * s;
+                    kv = kv * c - activated(to_float(kh[d + half]), act) * s;
                 } else {
-                    qv = qv * c + to_float(qh[i]) * s;
-                    kv = kv * c + to_float(kh[i]) * s;
+                    qv = qv * c + activated(to_float(qh[i]), act) * s;
+                    kv = kv * c + activated(to_float(kh[i]), act) * s;
                 }
             }
         }
@@ -100,7 +103,8 @@ constexpr int kFetchValues = 12; // ... and values
             const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * slice - 1);                 \
             const int t = idx / slice;                                                                                \
             const int c = min(v0 + idx - t * slice, vdim - 1);                                                        \
-            ahead_v[i] = to_float(proj[static_cast<size_t>(first + (from) + t) * ldp + v_off + head * vdim + c]);     \
+            ahead_v[i] = activated(                                                                                   \
+                to_float(proj[static_cast<size_t>(first + (from) + t) * ldp + v_off + head * vdim + c]), act);        \
         }                                                                                                             \
     }
 
@@ -109,7 +113,7 @@ __global__ void __launch_bounds__(512)
 retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* __restrict__ turned,
                  const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ seq_slot,
                  const int* __restrict__ q_start_loc, float* __restrict__ raw, long plane,
-                 int heads, int dim, int vdim, int slice, int slices, int groups, int padded, int chunk) {
+                 int heads, int dim, int vdim, int slice, int slices, int groups, int padded, int chunk, int act) {
     extern __shared__ float4 lds4[];
     float* lds = reinterpret_cast<float*>(lds4);
     const int rows = groups * DS;              // rows of the memory that this workgroup keeps
@@ -212,30 +216,38 @@ retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* _
 }
 #undef CIE_RETENTION_FETCH
 
-// o / sqrt(mean(o^2) over the head + eps) * silu(gate): one wave per (token, head)
+// o / sqrt(mean(o^2) + eps) [* weight] * gate: one wave per (token, run of `span` heads).  The mean runs over the
+// `span` heads of a run together (1: every head by itself; `heads`: all of a token's heads as one vector); `weight`
+// [heads * vdim] float32 or null; the gate is silu(g) (gate_act 0) or sigmoid(g) (1) of the projection's gate columns.
 template <typename T>
 __global__ void __launch_bounds__(256)
 retention_norm_kernel(float* __restrict__ raw, long plane, int parts, const T* __restrict__ proj, long ldp, int g_off,
-                      T* __restrict__ out, int tokens, int heads, int vdim, float eps) {
+                      T* __restrict__ out, int tokens, int heads, int vdim, float eps, int span,
+                      const float* __restrict__ weight, int gate_act) {
+    const int runs = heads / span;
     const int item = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-    if (item >= tokens * heads) return;  // (whole waves leave together)
+    if (item >= tokens * runs) return;  // (whole waves leave together)
     const int lane = threadIdx.x % kWave;
-    const int token = item / heads;
-    const int head = item - token * heads;
-    float* o = raw + static_cast<size_t>(token) * heads * vdim + head * vdim;
+    const int token = item / runs;
+    const int first = (item - token * runs) * span * vdim;  // the run's first column
+    const int width = span * vdim;
+    float* o = raw + static_cast<size_t>(token) * heads * vdim + first;
     float sum_sq = 0.f;
-    for (int c = lane; c < vdim; c += kWave) {
+    for (int c = lane; c < width; c += kWave) {
         float v = o[c];
         for (int p = 1; p < parts; ++p) v += o[static_cast<size_t>(p) * plane + c];  // (the parts in their order)
         o[c] = v;  // (this lane's own column: it reads it again below)
         sum_sq += v * v;
     }
-    const float inv = 1.0f / sqrtf(wave_sum(sum_sq) / static_cast<float>(vdim) + eps);
-    const T* gate = proj + static_cast<size_t>(token) * ldp + g_off + head * vdim;
-    T* dst = out + static_cast<size_t>(token) * heads * vdim + head * vdim;
-    for (int c = lane; c < vdim; c += kWave) {
+    const float inv = 1.0f / sqrtf(wave_sum(sum_sq) / static_cast<float>(width) + eps);
+    const T* gate = proj + static_cast<size_t>(token) * ldp + g_off + first;
+    T* dst = out + static_cast<size_t>(token) * heads * vdim + first;
+    for (int c = lane; c < width; c += kWave) {
         const float g = to_float(gate[c]);
-        dst[c] = from_float<T>((o[c] * inv) * (g * sigmoidf(g)));
+        const float open = gate_act == 1 ? sigmoidf(g) : g * sigmoidf(g);
+        float y = o[c] * inv;
+        if (weight) y *= weight[first + c];
+        dst[c] = from_float<T>(y * open);
     }
 }
 
@@ -243,10 +255,10 @@ template <typename T, int DS>
 int launch_retention(hipStream_t s, dim3 grid, int threads, size_t lds, const void* proj, long ldp, int v_off,
                      const float* turned, const float* decay, float* state, const int* seq_slot, const int* q_start_loc,
                      float* raw, long plane, int heads, int dim, int vdim, int slice, int slices, int groups, int padded,
-                     int chunk) {
+                     int chunk, int act) {
     retention_kernel<T, DS><<<grid, threads, lds, s>>>(static_cast<const T*>(proj), ldp, v_off, turned, decay, state,
                                                       seq_slot, q_start_loc, raw, plane, heads, dim, vdim, slice, slices,
-                                                      groups, padded, chunk);
+                                                      groups, padded, chunk, act);
     return cie_after_launch();
 }
 
@@ -365,7 +377,9 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
                           const float* cos_table, const float* sin_table, int rot, const float* decay, float* state,
                           const int* seq_slot, const int* positions, const int* q_start_loc, float* turned, float* raw,
                           void* out, int tokens, int sequences, int heads, int dim, int vdim, int rows_per_thread,
-                          int groups, int parts, int slice, int chunk, float eps, float key_scale) {
+                          int groups, int parts, int slice, int chunk, float eps, float key_scale, int act,
+                          int norm_span, const float* norm_weight, int gate_act) {
+    if (act < 0 || act > 1 || norm_span < 1 || heads % norm_span || gate_act < 0 || gate_act > 1) return CIE_BAD_ARGUMENT;
     if (sequences < 0 || tokens < 0 || heads <= 0 || heads > 65535 || dim <= 0 || vdim <= 0 || groups <= 0 || chunk <= 0 ||
         parts <= 0 || slice <= 0 || slice > vdim || rot < 0 || rot % 2 || rot > dim ||
         (rot > 0 && (!cos_table || !sin_table)) || !(eps > 0.f) ||
@@ -385,10 +399,10 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == CIE_F32)
         retention_turn_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(proj), ldp, q_off, k_off, cos_table,
-                                                           sin_table, rot, positions, turned, heads, dim, padded, key_scale);
+                                                           sin_table, rot, positions, turned, heads, dim, padded, key_scale, act);
     else if (dtype == CIE_BF16)
         retention_turn_kernel<bf16_t><<<tokens, 256, 0, s>>>(static_cast<const bf16_t*>(proj), ldp, q_off, k_off, cos_table,
-                                                            sin_table, rot, positions, turned, heads, dim, padded, key_scale);
+                                                            sin_table, rot, positions, turned, heads, dim, padded, key_scale, act);
     else
         return CIE_BAD_ARGUMENT;
     dim3 grid(sequences, heads, slices * parts);
@@ -396,7 +410,7 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
     int code = CIE_BAD_ARGUMENT;
 #define CIE_RETENTION(T, DS)                                                                                         \
     code = launch_retention<T, DS>(s, grid, threads, lds, proj, ldp, v_off, turned, decay, state, seq_slot,          \
-                                   q_start_loc, raw, plane, heads, dim, vdim, slice, slices, groups, padded, chunk)
+                                   q_start_loc, raw, plane, heads, dim, vdim, slice, slices, groups, padded, chunk, act)
     if (dtype == CIE_F32) {
         if (rows_per_thread == 4) CIE_RETENTION(float, 4);
         else if (rows_per_thread == 8) CIE_RETENTION(float, 8);
@@ -410,14 +424,16 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
     }
 #undef CIE_RETENTION
     if (code != CIE_OK) return code;
-    const int items = tokens * heads;
+    const int items = tokens * (heads / norm_span);
     const int blocks = (items + 3) / 4;
     if (dtype == CIE_F32)
         retention_norm_kernel<float><<<blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const float*>(proj), ldp, g_off,
-                                                           static_cast<float*>(out), tokens, heads, vdim, eps);
+                                                           static_cast<float*>(out), tokens, heads, vdim, eps, norm_span,
+                                                           norm_weight, gate_act);
     else
         retention_norm_kernel<bf16_t><<<blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const bf16_t*>(proj), ldp, g_off,
-                                                            static_cast<bf16_t*>(out), tokens, heads, vdim, eps);
+                                                            static_cast<bf16_t*>(out), tokens, heads, vdim, eps, norm_span,
+                                                            norm_weight, gate_act);
     return cie_after_launch();
 }
 

@@ -30,20 +30,98 @@ namespace {
 
 constexpr int kMaxExperts = 1024;
 
-// One wave ranks one token's logits z: its `top` experts and their scores to expert_out / weight_out (and the
-// experts to `copy` as well, where the caller wants them in LDS).
+// How a token's router outputs become a choice and weights.  Every step may be left out:
+//   s = sigmoid(z), or softmax(z) over all outputs                        (softmax)
+//   the choice ranks c = s + correction[e]                                (correction; without one and without the
+//                                                                          softmax the logits z themselves are ranked)
+//   the outputs form `groups` equal runs of neighbours; a run's score is its largest c, and only outputs of the
+//   `keep` best runs can be chosen                                        (groups > 1)
+//   weights w = s of the chosen, as they are, or divided by their sum + 1e-20 and times `scale`   (normalize)
+struct RouteShape {
+    int softmax;
+    const float* correction;  // [outputs] or null
+    int groups;               // <= 1: none (at most 64)
+    int keep;
+    int normalize;
+    float scale;
+};
+
+// One wave ranks one token's logits z: its `top` outputs and their weights to expert_out / weight_out (and the
+// outputs to `copy` as well, where the caller wants them in LDS).  Equal ranks: the lower index first.
 __device__ __forceinline__ void route_token(const float* __restrict__ z, int experts, int top, int lane,
                                             int* __restrict__ expert_out, float* __restrict__ weight_out,
-                                            int* copy) {
+                                            int* copy, const RouteShape shape) {
     constexpr int kMine = kMaxExperts / kWave;
-    float mine[kMine];
-    unsigned out = 0;  // bit i: expert lane + i * kWave is not there, or already chosen
+    float mine[kMine];   // what is ranked
+    float score[kMine];  // what becomes the weight
+    unsigned out = 0;  // bit i: expert lane + i * kWave is not there, or already chosen, or outside the kept runs
+    float z_max = -INFINITY;
 #pragma unroll
     for (int i = 0; i < kMine; ++i) {
         const int e = lane + i * kWave;
         mine[i] = e < experts ? z[e] : 0.f;  // (ranked by the logit: the score rises with it, and does not saturate)
         if (e >= experts) out |= 1u << i;
+        else z_max = fmaxf(z_max, mine[i]);
     }
+    const bool by_score = shape.softmax || shape.correction;
+    if (shape.softmax) {
+        z_max = wave_max(z_max);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) {
+            score[i] = (lane + i * kWave < experts) ? expf(mine[i] - z_max) : 0.f;
+            sum += score[i];
+        }
+        const float inv = 1.0f / wave_sum(sum);
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) score[i] *= inv;
+    } else {
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) score[i] = 1.0f / (1.0f + expf(-mine[i]));
+    }
+    if (by_score) {
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) {
+            const int e = lane + i * kWave;
+            mine[i] = score[i] + ((shape.correction && e < experts) ? shape.correction[e] : 0.f);
+        }
+    }
+    if (shape.groups > 1) {
+        // lane g holds run g's score; then the `keep` best runs, one after the other
+        const int per = experts / shape.groups;
+        float run_score = -INFINITY;
+        for (int g = 0; g < shape.groups; ++g) {
+            float best = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < kMine; ++i) {
+                const int e = lane + i * kWave;
+                if (e < experts && e / per == g) best = fmaxf(best, mine[i]);
+            }
+            best = wave_max(best);
+            if (lane == g) run_score = best;
+        }
+        unsigned long long kept = 0;
+        for (int k = 0; k < shape.keep; ++k) {
+            float best = run_score;
+            int best_g = (lane < shape.groups && !((kept >> lane) & 1ull)) ? lane : kWave;
+#pragma unroll
+            for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+                const float other = __shfl_xor(best, offset, kWave);
+                const int other_g = __shfl_xor(best_g, offset, kWave);
+                if (other_g != kWave && (best_g == kWave || other > best || (other == best && other_g < best_g))) {
+                    best = other;
+                    best_g = other_g;
+                }
+            }
+            if (best_g != kWave) kept |= 1ull << best_g;
+        }
+#pragma unroll
+        for (int i = 0; i < kMine; ++i) {
+            const int e = lane + i * kWave;
+            if (e < experts && !((kept >> (e / per)) & 1ull)) out |= 1u << i;
+        }
+    }
+    float total = 0.f;
     for (int k = 0; k < top; ++k) {
         float best = 0.f;
         int best_e = kMaxExperts;  // (none yet)
@@ -65,31 +143,43 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, int exp
                 best_e = other_e;
             }
         }
-        if (lane == 0) {
-            expert_out[k] = best_e;
-            weight_out[k] = 1.0f / (1.0f + expf(-best));
-            if (copy) copy[k] = best_e;
-        }
+        float chosen = 0.f;  // the score of the chosen one, from the lane that holds it
 #pragma unroll
         for (int i = 0; i < kMine; ++i)
-            if (lane + i * kWave == best_e) out |= 1u << i;
+            if (lane + i * kWave == best_e) {
+                out |= 1u << i;
+                chosen = score[i];
+            }
+        chosen = __shfl(chosen, best_e % kWave, kWave);
+        total += chosen;
+        if (lane == 0) {
+            expert_out[k] = best_e;
+            weight_out[k] = chosen;
+            if (copy) copy[k] = best_e;
+        }
+    }
+    if (shape.normalize && lane == 0) {
+        const float factor = shape.scale / (total + 1e-20f);
+        for (int k = 0; k < top; ++k) weight_out[k] *= factor;  // (this thread's own stores)
     }
 }
 
 // One wave per token.
 __global__ void __launch_bounds__(256)
 route_kernel(const float* __restrict__ logits, int tokens, int experts, int top, int* __restrict__ pair_expert,
-             float* __restrict__ pair_weight) {
+             float* __restrict__ pair_weight, RouteShape shape) {
     const int lane = threadIdx.x % kWave;
     const int token = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
     if (token >= tokens) return;
     route_token(logits + static_cast<size_t>(token) * experts, experts, top, lane,
-                pair_expert + static_cast<size_t>(token) * top, pair_weight + static_cast<size_t>(token) * top, nullptr);
+                pair_expert + static_cast<size_t>(token) * top, pair_weight + static_cast<size_t>(token) * top, nullptr,
+                shape);
 }
 
 // One workgroup.  sorted[i]: the pair at place i of the order by expert; tiles (expert, first place, rows).
-// (pair_expert may lie in LDS.)
-__device__ __forceinline__ void arrange_pairs(const int* pair_expert, int pairs, int experts, int tile_rows,
+// (pair_expert may lie in LDS.)  Only the first `real` of the `experts` router outputs have weights and get tiles:
+// the pairs of the others stand at the end of the order, and whoever owns them fills their rows.
+__device__ __forceinline__ void arrange_pairs(const int* pair_expert, int pairs, int experts, int real, int tile_rows,
                                               int* __restrict__ sorted, int* __restrict__ tile_expert,
                                               int* __restrict__ tile_begin, int* __restrict__ tile_count,
                                               int* __restrict__ n_tiles) {
@@ -110,12 +200,12 @@ __device__ __forceinline__ void arrange_pairs(const int* pair_expert, int pairs,
             first[e] = place;
             first_tile[e] = tile;
             place += count[e];
-            tile += (count[e] + tile_rows - 1) / tile_rows;
+            if (e < real) tile += (count[e] + tile_rows - 1) / tile_rows;
         }
         *n_tiles = tile;
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+    for (int e = threadIdx.x; e < real; e += blockDim.x) {
         const int tiles = (count[e] + tile_rows - 1) / tile_rows;
         for (int t = 0; t < tiles; ++t) {
             tile_expert[first_tile[e] + t] = e;
@@ -132,10 +222,10 @@ __device__ __forceinline__ void arrange_pairs(const int* pair_expert, int pairs,
 }
 
 __global__ void __launch_bounds__(1024)
-arrange_kernel(const int* __restrict__ pair_expert, int pairs, int experts, int tile_rows, int* __restrict__ sorted,
-               int* __restrict__ tile_expert, int* __restrict__ tile_begin, int* __restrict__ tile_count,
-               int* __restrict__ n_tiles) {
-    arrange_pairs(pair_expert, pairs, experts, tile_rows, sorted, tile_expert, tile_begin, tile_count, n_tiles);
+arrange_kernel(const int* __restrict__ pair_expert, int pairs, int experts, int real, int tile_rows,
+               int* __restrict__ sorted, int* __restrict__ tile_expert, int* __restrict__ tile_begin,
+               int* __restrict__ tile_count, int* __restrict__ n_tiles) {
+    arrange_pairs(pair_expert, pairs, experts, real, tile_rows, sorted, tile_expert, tile_begin, tile_count, n_tiles);
 }
 
 // Few tokens (a step of up to sixteen single tokens): choice and order in one workgroup, one launch (beyond that
@@ -145,18 +235,18 @@ constexpr int kFusedPairs = 1024;
 constexpr int kFusedTokens = 16;
 
 __global__ void __launch_bounds__(1024)
-route_arrange_kernel(const float* __restrict__ logits, int tokens, int experts, int top,
+route_arrange_kernel(const float* __restrict__ logits, int tokens, int experts, int real, int top,
                      int* __restrict__ pair_expert, float* __restrict__ pair_weight, int tile_rows,
                      int* __restrict__ sorted, int* __restrict__ tile_expert, int* __restrict__ tile_begin,
-                     int* __restrict__ tile_count, int* __restrict__ n_tiles) {
+                     int* __restrict__ tile_count, int* __restrict__ n_tiles, RouteShape shape) {
     __shared__ int chosen[kFusedPairs];
     const int lane = threadIdx.x % kWave;
     for (int token = threadIdx.x / kWave; token < tokens; token += blockDim.x / kWave)
         route_token(logits + static_cast<size_t>(token) * experts, experts, top, lane,
                     pair_expert + static_cast<size_t>(token) * top, pair_weight + static_cast<size_t>(token) * top,
-                    chosen + token * top);
+                    chosen + token * top, shape);
     __syncthreads();
-    arrange_pairs(chosen, tokens * top, experts, tile_rows, sorted, tile_expert, tile_begin, tile_count, n_tiles);
+    arrange_pairs(chosen, tokens * top, experts, real, tile_rows, sorted, tile_expert, tile_begin, tile_count, n_tiles);
 }
 
 struct ExpertArgs {
@@ -221,7 +311,7 @@ experts_gate_up_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restri
         const int row = rt * 16 + r;
         const int pair = a.sorted[begin + min(row, rows - 1)];
         x_row[rt] = x + static_cast<size_t>(pair / a.top) * K;
-        weight[rt] = row < rows ? a.pair_weight[pair] : 0.f;
+        weight[rt] = row < rows ? (a.pair_weight ? a.pair_weight[pair] : 1.f) : 0.f;
     }
     floatx4 acc_g[RT], acc_u[RT];
 #pragma unroll
@@ -381,7 +471,7 @@ experts_gather_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xs, con
                       const float* __restrict__ pair_weight, int pairs, int top, int hidden) {
     const int place = blockIdx.x;
     const int pair = sorted[place];
-    const float w = pair_weight[pair];
+    const float w = pair_weight ? pair_weight[pair] : 1.f;
     const bf16_t* src = x + static_cast<size_t>(pair / top) * hidden;
     bf16_t* dst = xs + static_cast<size_t>(place) * hidden;
     for (int k = threadIdx.x * 8; k < hidden; k += blockDim.x * 8) {
@@ -546,7 +636,7 @@ experts_gate_up_plain_kernel(const T* __restrict__ x, const T* __restrict__ w_ga
     const int expert = a.tile_expert[tile];
     const int place = a.tile_begin[tile] + row;
     const int pair = a.sorted[place];
-    const float w = a.pair_weight[pair];
+    const float w = a.pair_weight ? a.pair_weight[pair] : 1.f;
     const int K = a.hidden;
     const T* x_row = x + static_cast<size_t>(pair / a.top) * K;
     const T* wg = w_gate_up + (static_cast<size_t>(expert) * 2 * a.ff + col) * K;
@@ -578,25 +668,59 @@ experts_down_plain_kernel(const T* __restrict__ act, const T* __restrict__ w_dow
     parts[static_cast<size_t>(a.sorted[place]) * a.hidden + col] = sum;
 }
 
+// parts[p, :] = x[token(p), :] for every pair whose choice is one of the outputs behind the `real` experts (an
+// expert that hands its input on); the other pairs' rows are the down product's.
+template <typename T>
+__global__ void __launch_bounds__(256)
+experts_identity_kernel(const T* __restrict__ x, const int* __restrict__ pair_expert, int real,
+                        float* __restrict__ parts, int top, int hidden) {
+    const int pair = blockIdx.x;
+    if (pair_expert[pair] < real) return;
+    const T* src = x + static_cast<size_t>(pair / top) * hidden;
+    float* dst = parts + static_cast<size_t>(pair) * hidden;
+    for (int k = threadIdx.x; k < hidden; k += blockDim.x) dst[k] = to_float(src[k]);
+}
+
 }  // namespace
 
+CIE_API int cie_experts_identity(void* stream, int dtype, const void* x, const int* pair_expert, int real, float* parts,
+                                 int pairs, int top, int hidden) {
+    if (pairs < 0 || top < 1 || hidden < 1 || real < 0) return CIE_BAD_ARGUMENT;
+    if (pairs == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == CIE_F32)
+        experts_identity_kernel<float><<<pairs, 256, 0, s>>>(static_cast<const float*>(x), pair_expert, real, parts, top, hidden);
+    else if (dtype == CIE_BF16)
+        experts_identity_kernel<bf16_t><<<pairs, 256, 0, s>>>(static_cast<const bf16_t*>(x), pair_expert, real, parts, top, hidden);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+// `experts` router outputs of which the first `real` are experts with weights (the others hand their input on: their
+// pairs get no tiles).  The choice's shape: see RouteShape.
 CIE_API int cie_experts_route(void* stream, const float* logits, int tokens, int experts, int top, int tile_rows,
                               int* pair_expert, float* pair_weight, int* sorted, int* tile_expert, int* tile_begin,
-                              int* tile_count, int* n_tiles) {
-    if (tokens < 0 || experts < 1 || experts > kMaxExperts || top < 1 || top > experts || tile_rows < 1)
+                              int* tile_count, int* n_tiles, int real, int softmax, const float* correction,
+                              int groups, int keep, int normalize, float scale) {
+    if (tokens < 0 || experts < 1 || experts > kMaxExperts || top < 1 || top > experts || tile_rows < 1 || real < 0 ||
+        real > experts)
         return CIE_BAD_ARGUMENT;
+    if (groups > 1 && (groups > kWave || experts % groups || keep < 1 || keep > groups || top > keep * (experts / groups)))
+        return CIE_BAD_ARGUMENT;
+    const RouteShape shape{softmax, correction, groups, keep, normalize, scale};
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (tokens > 0 && tokens <= kFusedTokens && tokens * top <= kFusedPairs) {
-        route_arrange_kernel<<<1, 1024, 0, s>>>(logits, tokens, experts, top, pair_expert, pair_weight, tile_rows, sorted,
-                                                tile_expert, tile_begin, tile_count, n_tiles);
+        route_arrange_kernel<<<1, 1024, 0, s>>>(logits, tokens, experts, real, top, pair_expert, pair_weight, tile_rows,
+                                                sorted, tile_expert, tile_begin, tile_count, n_tiles, shape);
         return cie_after_launch();
     }
     if (tokens > 0) {
-        route_kernel<<<(tokens + 3) / 4, 256, 0, s>>>(logits, tokens, experts, top, pair_expert, pair_weight);
+        route_kernel<<<(tokens + 3) / 4, 256, 0, s>>>(logits, tokens, experts, top, pair_expert, pair_weight, shape);
         if (hipGetLastError() != hipSuccess) return CIE_LAUNCH_FAILED;
     }
-    arrange_kernel<<<1, 1024, 0, s>>>(pair_expert, tokens * top, experts, tile_rows, sorted, tile_expert, tile_begin,
-                                      tile_count, n_tiles);
+    arrange_kernel<<<1, 1024, 0, s>>>(pair_expert, tokens * top, experts, real, tile_rows, sorted, tile_expert,
+                                      tile_begin, tile_count, n_tiles);
     return cie_after_launch();
 }
 

@@ -930,6 +930,8 @@ def latent_rows(proj: torch.Tensor, weight: torch.Tensor, heads: int, plain: int
 RETENTION_ROWS = (4, 8, 16, 32)  # rows of a head's memory that one thread keeps in registers
 RETENTION_SLICE = 64             # value columns of a head that one workgroup takes
 RETENTION_LDS_FLOATS = 15 * 1024
+RETENTION_ACTIVATIONS = {None: 0, "silu": 1}   # what queries, keys and values pass through on their way in
+RETENTION_GATES = {"silu": 0, "sigmoid": 1}    # the function of the gate columns that multiplies the read-out
 
 
 def plan_retention(dim: int, vdim: int, units: int = 1) -> tuple[int, int, int, int, int]:
@@ -964,12 +966,24 @@ def plan_retention(dim: int, vdim: int, units: int = 1) -> tuple[int, int, int, 
 def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optional[torch.Tensor],
               sin: Optional[torch.Tensor], rot: int, decay: torch.Tensor, state: torch.Tensor, seq_slot: torch.Tensor,
               positions: torch.Tensor, q_start_loc: torch.Tensor, sequences: int, heads: int, dim: int, vdim: int,
-              eps: float, key_scale: float, longest_position: int) -> torch.Tensor:
+              eps: float, key_scale: float, longest_position: int, activation: Optional[str] = None,
+              norm_span: int = 1, norm_weight: Optional[torch.Tensor] = None, gate: str = "silu") -> torch.Tensor:
     """Retention over a step's tokens (``csrc/recurrent.hip``; ``positions`` int32 [T] are the tokens' own).
     ``proj`` [T, ...] holds each token's queries, keys
     (heads x dim), values and gates (heads x vdim) from the columns ``offsets`` on; ``state`` float32
     [slots, heads, dim, vdim] is read and written at the sequences' slots; cos/sin float32 [positions, rot/2]
-    must reach ``longest_position``.  Returns [T, heads * vdim] in ``proj``'s type."""
+    must reach ``longest_position``.  ``activation="silu"``: queries, keys and values pass through silu on their way
+    in.  The read-out is divided by its root mean square over runs of ``norm_span`` heads (1: each head alone;
+    ``heads``: the token's whole row), multiplied by ``norm_weight`` (float32 [heads * vdim]) where given, and by
+    ``silu`` or ``sigmoid`` (``gate``) of the gate columns.  Returns [T, heads * vdim] in ``proj``'s type."""
+    if activation not in RETENTION_ACTIVATIONS or gate not in RETENTION_GATES:
+        raise ValueError(f"activation is one of {list(RETENTION_ACTIVATIONS)}, gate one of {list(RETENTION_GATES)}")
+    if norm_span < 1 or heads % norm_span:
+        raise ValueError(f"the norm's runs of {norm_span} heads do not divide {heads} heads")
+    if norm_weight is not None:
+        _gpu("norm_weight", norm_weight, torch.float32, 1)
+        if norm_weight.shape[0] != heads * vdim:
+            raise ValueError(f"norm_weight must be [{heads * vdim}], is {tuple(norm_weight.shape)}")
     if not (proj.is_cuda and proj.dim() == 2 and proj.stride(1) == 1 and proj.dtype in _CODES):
         raise ValueError("proj must be a float32 or bfloat16 GPU matrix with unit inner stride")
     tokens = proj.shape[0]
@@ -999,7 +1013,8 @@ def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optio
         _stream(), _i(_code(proj.dtype)), _ptr(proj), ldp, _i(q_off), _i(k_off), _i(v_off), _i(g_off),
         _ptr(cos if rot else None), _ptr(sin if rot else None), _i(rot), _ptr(decay), _ptr(state), _ptr(seq_slot),
         _ptr(positions), _ptr(q_start_loc), _ptr(turned), _ptr(raw), _ptr(out), _i(tokens), _i(sequences), _i(heads), _i(dim), _i(vdim),
-        _i(rows), _i(groups), _i(parts), _i(piece), _i(chunk), _f(eps), _f(key_scale)))
+        _i(rows), _i(groups), _i(parts), _i(piece), _i(chunk), _f(eps), _f(key_scale),
+        _i(RETENTION_ACTIVATIONS[activation]), _i(norm_span), _ptr(norm_weight), _i(RETENTION_GATES[gate])))
     return out
 
 
@@ -1104,6 +1119,56 @@ def branch_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weig
     return rows
 
 
+def group_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor, groups: int, eps: float,
+                   out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, branch_gate: Optional[torch.Tensor] = None,
+                   parts: Optional[torch.Tensor] = None, part_weight: Optional[torch.Tensor] = None,
+                   plus: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``residual += branch * sigmoid(branch_gate) + sum_p part_weight[:, p] * parts[:, p] + plus`` (whatever of it
+    is given; float32, in place unless ``rows``), then the RMS norm of every row in ``groups`` equal consecutive
+    parts, each over its own root mean square, the whole times ``weight`` (float32 [H]).  ``branch`` [T, H] float32
+    or ``out_dtype``; ``branch_gate`` float32 [T] (logits); ``parts`` float32 [T, P, H]; ``part_weight`` float32
+    [T, P]; ``plus`` float32 [T, H].  With ``rows`` (int32 [n]) only those rows come back, in that order."""
+    _gpu("residual", residual, torch.float32, 2)
+    tokens, hidden = residual.shape
+    _gpu("weight", weight, torch.float32, 1)
+    if not (weight.shape[0] == hidden and hidden + groups <= MAX_NORM_WIDTH and eps > 0):
+        raise ValueError(f"weight {tuple(weight.shape)}, hidden {hidden}, eps {eps} do not fit the norm kernel")
+    if groups < 1 or hidden % groups:
+        raise ValueError(f"{groups} groups do not divide a row of {hidden}")
+    if branch is not None:
+        _gpu("branch", branch, dims=2)
+        if not (branch.shape == residual.shape and branch.dtype in (torch.float32, out_dtype)):
+            raise ValueError(f"branch {tuple(branch.shape)} {branch.dtype} does not fit {tuple(residual.shape)} {out_dtype}")
+    if branch_gate is not None:
+        _gpu("branch_gate", branch_gate, torch.float32, 1)
+        if branch is None or branch_gate.shape[0] != tokens:
+            raise ValueError("a gate comes with a branch, one logit per row")
+    n_parts = 0
+    if parts is not None:
+        _gpu("parts", parts, torch.float32, 3)
+        if not (parts.shape[0] == tokens and parts.shape[2] == hidden):
+            raise ValueError(f"parts {tuple(parts.shape)} do not fit {tuple(residual.shape)}")
+        n_parts = parts.shape[1]
+    if part_weight is not None:
+        _gpu("part_weight", part_weight, torch.float32)
+        if parts is None or part_weight.numel() != tokens * n_parts:
+            raise ValueError("part weights come with parts, one per part and row")
+    if plus is not None:
+        _gpu("plus", plus, torch.float32, 2)
+        if plus.shape != residual.shape:
+            raise ValueError(f"plus {tuple(plus.shape)} vs residual {tuple(residual.shape)}")
+    n_out = tokens
+    if rows is not None:
+        _gpu("rows", rows, torch.int32, 1)
+        n_out = rows.shape[0]
+    out = torch.empty((n_out, hidden), dtype=out_dtype, device=residual.device)
+    _run("cie_group_norm_add", load_library().cie_group_norm_add(
+        _stream(), _i(_code(branch.dtype if branch is not None else out_dtype)), _i(_code(out_dtype)), _ptr(residual),
+        _ptr(branch), _ptr(branch_gate), _ptr(parts), _ptr(part_weight), _i(n_parts), _ptr(plus), _ptr(weight),
+        _ptr(out), _ptr(rows), _i(n_out), _i(hidden), _i(groups), _f(eps)))
+    return out
+
+
 def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, offset: float) -> torch.Tensor:
     """``g * sigmoid(alpha * g) * (u + offset)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)`` for
     gate_up [T, 2I] (gate half first)."""
@@ -1146,12 +1211,15 @@ def heads_prepare(proj: torch.Tensor, offsets: tuple[int, int, int], q_heads: in
                   k_weight: Optional[torch.Tensor], eps: float, temperature: Optional[tuple[float, int]],
                   positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor,
                   block_table: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, tokens: int,
-                  write_kv: bool = True) -> torch.Tensor:
+                  write_kv: bool = True, rotary: Optional[tuple] = None) -> torch.Tensor:
     """From projected rows ``proj`` [T, >= ...] (queries at column ``offsets[0]``, keys at ``offsets[1]``, values at
     ``offsets[2]``, heads of ``dim`` / ``dim`` / ``vdim`` numbers) to queries ``[T, q_heads * kernel_dim]`` and the
     token's cache entries: per-head RMS norm of queries and keys (``norm``: ``None``, ``"unit"`` or ``"weight"`` with
     float32 weights [dim]), the queries times ``1 + coef * ln(floor((p + 1) / every) + 1)`` (``temperature = (coef,
-    every)``), heads zero-padded up to the kernels' sizes."""
+    every)``), heads zero-padded up to the kernels' sizes.  ``rotary = (cos, sin, rot, neighbours)``: after the norm
+    the first ``rot`` numbers of every query and key head turn by the token's position, in pairs of neighbours
+    ``(2i, 2i + 1)`` or of the halves ``(i, i + rot / 2)``; cos and sin are float32 ``[positions, rot / 2]`` and must
+    reach every position of the step (the caller sees to that)."""
     if not (proj.is_cuda and proj.dim() == 2 and proj.stride(1) == 1):
         raise ValueError("proj must be 2-d on the GPU with unit inner stride")
     dtype = proj.dtype
@@ -1180,17 +1248,29 @@ def heads_prepare(proj: torch.Tensor, offsets: tuple[int, int, int], q_heads: in
     coef, every = temperature if temperature else (0.0, 0)
     if temperature and every < 1:
         raise ValueError("the temperature's period must be positive")
+    cos = sin = None
+    rot, neighbours = 0, False
+    if rotary is not None:
+        cos, sin, rot, neighbours = rotary
+        if rot < 2 or rot % 2 or rot > dim:
+            raise ValueError(f"{rot} turning numbers in heads of {dim}: even, at least 2, at most the head")
+        for name, table in (("cos", cos), ("sin", sin)):
+            _gpu(name, table, torch.float32, 2)
+            if table.shape[1] != rot // 2 or not table.is_contiguous():
+                raise ValueError(f"{name} {tuple(table.shape)} does not hold {rot // 2} pairs per position")
     q_out = torch.empty((tokens, q_heads * kernel_dim), dtype=dtype, device=proj.device)
     _run("cie_heads_prepare", load_library().cie_heads_prepare(
         _stream(), _i(_code(dtype)), _ptr(proj), _i(proj.stride(0)), _i(q_off), _i(k_off), _i(v_off), _ptr(q_weight),
         _ptr(k_weight), _i(NORM_MODES[norm]), _f(eps), _f(coef), _i(every), _ptr(positions), _ptr(seq_of_token),
         _ptr(seq_slot), _ptr(block_table), _i(block_table.shape[1]), _ptr(q_out), _ptr(k_pool), _ptr(v_pool),
         _i(tokens), _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(kernel_dim), _i(kernel_vdim), _i(page_size),
-        _i(1 if write_kv else 0)))
+        _i(1 if write_kv else 0), _ptr(cos), _ptr(sin), _i(rot), _i(1 if neighbours else 0)))
     return q_out
 
 
-def _check_score_shape(q_heads: int, slopes, sinks, softcap) -> None:
+def _check_score_shape(q_heads: int, slopes, sinks, softcap, window=None, chunk=None) -> None:
+    if chunk is not None and (chunk < 1 or window):
+        raise ValueError(f"chunks hold at least one token and stand in a window's place, got chunk {chunk}, window {window}")
     for name, t in (("slopes", slopes), ("sinks", sinks)):
         if t is not None:
             _gpu(name, t, torch.float32, 1)
@@ -1213,8 +1293,10 @@ def scored_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torc
                              positions: torch.Tensor, seq_of_token: torch.Tensor, seq_slot: torch.Tensor, tokens: int,
                              q_heads: int, kv_heads: int, dim: int, vdim: int, window: Optional[int], scale: float,
                              softcap: Optional[float] = None, slopes: Optional[torch.Tensor] = None,
-                             sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Attention of each token over its request's cached keys with shaped scores (see ``csrc/attention_scored.hip``):
+                             sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                             chunk: Optional[int] = None) -> torch.Tensor:
+    """Attention of each token over its request's cached keys with shaped scores (see ``csrc/attention_scored.hip``;
+    ``chunk``: a token sees the keys of its own chunk of that many positions, counted from position 0, up to itself):
     ``q`` [T, q_heads * dim]; returns [T, q_heads * vdim].  ``gate`` [T, >= q_heads] (a view is fine): head h's output
     is multiplied by ``sigmoid(gate[t, h])``.  float32 or bfloat16."""
     _gpu("q", q, dims=2)
@@ -1228,14 +1310,14 @@ def scored_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torc
         if not (meta.shape[0] >= tokens):
             raise ValueError(f"{name} has {meta.shape[0]} entries for {tokens} tokens")
     _gpu("seq_slot", seq_slot, torch.int32, 1)
-    _check_score_shape(q_heads, slopes, sinks, softcap)
+    _check_score_shape(q_heads, slopes, sinks, softcap, window, chunk)
     gate_stride = _check_gate(gate, tokens, q_heads, q.dtype)
     out = torch.empty((tokens, q_heads * vdim), dtype=q.dtype, device=q.device)
     _run("cie_scored_attention_generic", load_library().cie_scored_attention_generic(
         _stream(), _i(_code(q.dtype)), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _i(block_table.shape[1]),
         _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(gate), _i(gate_stride), _ptr(out), _i(tokens),
         _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(page_size), _i(window or 0), _f(scale), _f(softcap or 0.0),
-        _ptr(slopes), _ptr(sinks)))
+        _ptr(slopes), _ptr(sinks), _i(chunk or 0)))
     return out
 
 
@@ -1246,7 +1328,7 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
                           tokens_per_tile: int, row_tiles: int, window: Optional[int], scale: float,
                           softcap: Optional[float] = None, slopes: Optional[torch.Tensor] = None,
                           sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                          n_splits: int = 1, keys_per_split: int = 0) -> torch.Tensor:
+                          n_splits: int = 1, keys_per_split: int = 0, chunk: Optional[int] = None) -> torch.Tensor:
     """The same on the matrix cores (bfloat16, (dim, vdim) in ``SCORED_MFMA_DIMS``, pages of a power of two >= 4):
     tiles of ``tokens_per_tile`` consecutive tokens of one sequence (``tile_seq``, ``tile_q0`` int32 [n_tiles]; both
     ``None``: tile i is sequence i's first), whose rows times the heads per key head fill ``row_tiles`` tiles of 16.
@@ -1277,7 +1359,7 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
             raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
     if tile_seq is None and n_tiles > sequences:
         raise ValueError(f"{n_tiles} tiles for {sequences} sequences")
-    _check_score_shape(q_heads, slopes, sinks, softcap)
+    _check_score_shape(q_heads, slopes, sinks, softcap, window, chunk)
     gate_stride = _check_gate(gate, tokens, q_heads, q.dtype)
     out = torch.empty((tokens, q_heads * vdim), dtype=q.dtype, device=q.device)
     part_o = part_ml = None
@@ -1294,7 +1376,7 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
         _ptr(tile_q0), _i(n_tiles), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len), _ptr(q_start_loc), _ptr(gate),
         _i(gate_stride), _ptr(out), _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(page_size), _i(tokens_per_tile),
         _i(row_tiles), _i(window or 0), _f(scale), _f(softcap or 0.0), _ptr(slopes), _ptr(sinks), _i(n_splits),
-        _i(keys_per_split), _ptr(part_o), _ptr(part_ml)))
+        _i(keys_per_split), _ptr(part_o), _ptr(part_ml), _i(chunk or 0)))
     return out
 
 
@@ -1307,22 +1389,46 @@ class ExpertRoute:
     """What ``experts_route`` leaves on the device for the expert products of one step."""
 
     __slots__ = ("pair_expert", "pair_weight", "sorted", "tile_expert", "tile_begin", "tile_count", "n_tiles",
-                 "max_tiles", "tile_rows", "top", "pairs")
+                 "max_tiles", "tile_rows", "top", "pairs", "real", "pair_expert_outputs")
 
 
-def experts_route(logits: torch.Tensor, top: int, tile_rows: int = 16) -> ExpertRoute:
+MAX_EXPERT_GROUPS = 64
+
+
+def experts_route(logits: torch.Tensor, top: int, tile_rows: int = 16, real: Optional[int] = None,
+                  scoring: str = "sigmoid", correction: Optional[torch.Tensor] = None,
+                  groups: Optional[tuple[int, int]] = None, normalize: bool = False, scale: float = 1.0) -> ExpertRoute:
     """Scores ``sigmoid(logits)`` (float32 [T, E]), the ``top`` largest per token (ranked by the logits, which order
     the scores and do not saturate; lowest index first among equals),
     and the (token, choice) pairs sorted by expert in tiles of at most ``tile_rows`` rows.  Nothing comes back to
-    the host: grids are sized for ``max_tiles`` and the kernels read the true count."""
+    the host: grids are sized for ``max_tiles`` and the kernels read the true count.
+
+    What else a router may ask for: ``scoring="softmax"`` (scores are the softmax over all E outputs);
+    ``correction`` (float32 [E], added to the scores for the choice only); ``groups=(count, keep)`` (the outputs form
+    ``count`` equal runs of neighbours, a run counts by its largest choice score, and only outputs of the ``keep``
+    best runs can be chosen); ``normalize`` (the chosen scores divided by their sum + 1e-20, times ``scale``);
+    ``real`` (only the first ``real`` outputs are experts with weights: pairs of the others get no tiles, and
+    ``experts_forward`` hands their token's row on as it is)."""
     _gpu("logits", logits, torch.float32, 2)
     tokens, experts = logits.shape
     if not (1 <= top <= experts <= MAX_EXPERTS and tile_rows >= 1):
         raise ValueError(f"{top} of {experts} experts (at most {MAX_EXPERTS}) in tiles of {tile_rows}")
+    real = experts if real is None else real
+    if not 0 <= real <= experts or scoring not in ("sigmoid", "softmax"):
+        raise ValueError(f"{real} experts of {experts} outputs with {scoring!r} scores")
+    if correction is not None:
+        _gpu("correction", correction, torch.float32, 1)
+        if correction.shape[0] != experts:
+            raise ValueError(f"correction must be [{experts}], is {tuple(correction.shape)}")
+    count, keep = groups if groups else (1, 1)
+    if count > 1 and not (count <= MAX_EXPERT_GROUPS and experts % count == 0 and 1 <= keep <= count
+                          and top <= keep * (experts // count)):
+        raise ValueError(f"{count} groups of which {keep} are kept do not fit {top} of {experts} outputs")
     route = ExpertRoute()
     pairs = tokens * top
-    route.pairs, route.top, route.tile_rows = pairs, top, tile_rows
-    route.max_tiles = min(pairs, pairs // tile_rows + experts)
+    route.pairs, route.top, route.tile_rows, route.real = pairs, top, tile_rows, real
+    route.pair_expert_outputs = experts  # how many outputs the router has; those from ``real`` on have no weights
+    route.max_tiles = min(pairs, pairs // tile_rows + real)
     ints = torch.empty(2 * pairs + 3 * max(route.max_tiles, 1) + 1, dtype=torch.int32, device=logits.device)
     route.pair_expert, route.sorted = ints[:pairs], ints[pairs: 2 * pairs]
     base = 2 * pairs
@@ -1333,14 +1439,17 @@ def experts_route(logits: torch.Tensor, top: int, tile_rows: int = 16) -> Expert
     _run("cie_experts_route", load_library().cie_experts_route(
         _stream(), _ptr(logits), _i(tokens), _i(experts), _i(top), _i(tile_rows), _ptr(route.pair_expert),
         _ptr(route.pair_weight), _ptr(route.sorted), _ptr(route.tile_expert), _ptr(route.tile_begin),
-        _ptr(route.tile_count), _ptr(route.n_tiles)))
+        _ptr(route.tile_count), _ptr(route.n_tiles), _i(real), _i(1 if scoring == "softmax" else 0), _ptr(correction),
+        _i(count), _i(keep), _i(1 if normalize else 0), _f(scale)))
     return route
 
 
 def experts_forward(x: torch.Tensor, route: ExpertRoute, w_gate_up: torch.Tensor, w_down: torch.Tensor, limit: float,
-                    alpha: float, offset: float, mfma: bool) -> torch.Tensor:
+                    alpha: float, offset: float, mfma: bool, weight_input: bool = True) -> torch.Tensor:
     """The chosen experts' outputs, float32 ``[T, top, hidden]``: row (t, k) is expert ``k`` of token t run on
-    ``weight * x[t]``.  ``w_gate_up`` [E, 2 * ff, hidden] (gate rows first), ``w_down`` [E, hidden, ff]."""
+    ``weight * x[t]``, or, with ``weight_input=False``, on ``x[t]`` itself (whoever sums the rows then applies
+    ``route.pair_weight``).  ``w_gate_up`` [E, 2 * ff, hidden] (gate rows first), ``w_down`` [E, hidden, ff].  A pair
+    whose choice lies behind the experts that have weights (``route.real``) gets ``x[t]`` as its row."""
     _gpu("x", x, dims=2)
     tokens, hidden = x.shape
     _gpu("w_gate_up", w_gate_up, x.dtype, 3)
@@ -1348,7 +1457,7 @@ def experts_forward(x: torch.Tensor, route: ExpertRoute, w_gate_up: torch.Tensor
     experts, twice, _ = w_gate_up.shape
     ff = twice // 2
     if not (w_gate_up.shape == (experts, 2 * ff, hidden) and w_down.shape == (experts, hidden, ff)
-            and tokens * route.top == route.pairs):
+            and tokens * route.top == route.pairs and experts == route.real):
         raise ValueError(f"expert weights {tuple(w_gate_up.shape)}, {tuple(w_down.shape)} do not fit rows {tuple(x.shape)}")
     if mfma and not (x.dtype == torch.bfloat16 and hidden % 8 == 0 and ff % 8 == 0 and route.tile_rows in EXPERT_TILE_ROWS):
         raise ValueError("the matrix-core form takes bfloat16, widths that are multiples of 8 and tiles of 16, 32, 64 or 128 rows")
@@ -1357,19 +1466,25 @@ def experts_forward(x: torch.Tensor, route: ExpertRoute, w_gate_up: torch.Tensor
     act = torch.empty((route.pairs, ff), dtype=x.dtype, device=x.device)
     parts = torch.empty((tokens, route.top, hidden), dtype=torch.float32, device=x.device)
     lib = load_library()
+    rows_in = x
+    pair_weight = route.pair_weight if weight_input else None
     if mfma and route.tile_rows == 128:
         # many rows an expert: the rows in sorted order, weights applied, for the form that stages tiles through LDS
         gathered = torch.empty((route.pairs, hidden), dtype=x.dtype, device=x.device)
         _run("cie_experts_gather", lib.cie_experts_gather(_stream(), _ptr(x), _ptr(gathered), _ptr(route.sorted),
-                                                          _ptr(route.pair_weight), _i(route.pairs), _i(route.top), _i(hidden)))
+                                                          _ptr(pair_weight), _i(route.pairs), _i(route.top), _i(hidden)))
         x = gathered
     _run("cie_experts_gate_up", lib.cie_experts_gate_up(
         _stream(), _i(_code(x.dtype)), _i(1 if mfma else 0), _ptr(x), _ptr(w_gate_up), _ptr(act), _ptr(route.sorted),
-        _ptr(route.pair_weight), _ptr(route.tile_expert), _ptr(route.tile_begin), _ptr(route.tile_count),
+        _ptr(pair_weight), _ptr(route.tile_expert), _ptr(route.tile_begin), _ptr(route.tile_count),
         _ptr(route.n_tiles), _i(route.max_tiles), _i(route.tile_rows), _i(route.top), _i(hidden), _i(ff), _f(limit),
         _f(alpha), _f(offset)))
     _run("cie_experts_down", lib.cie_experts_down(
         _stream(), _i(_code(x.dtype)), _i(1 if mfma else 0), _ptr(act), _ptr(w_down), _ptr(parts), _ptr(route.sorted),
         _ptr(route.tile_expert), _ptr(route.tile_begin), _ptr(route.tile_count), _ptr(route.n_tiles),
         _i(route.max_tiles), _i(route.tile_rows), _i(route.top), _i(hidden), _i(ff)))
+    if route.real < route.pair_expert_outputs:
+        _run("cie_experts_identity", lib.cie_experts_identity(
+            _stream(), _i(_code(rows_in.dtype)), _ptr(rows_in), _ptr(route.pair_expert), _i(route.real), _ptr(parts),
+            _i(route.pairs), _i(route.top), _i(hidden)))
     return parts

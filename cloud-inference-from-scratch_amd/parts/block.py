@@ -36,8 +36,12 @@ class PreNormBlock:
         self.mixer = build_part("mixer", spec.mixer)
         self.norm2 = build_part("norm", spec.norm2)
         self.feed_forward = build_part("feed_forward", spec.feed_forward)
+        # a layer without feed-forward has no second norm (a checkpoint that holds one all the same is accepted)
+        self.has_feed_forward = spec.feed_forward.kind != "none"
 
     def _parts(self):
+        if not self.has_feed_forward:
+            return (("norm1", self.norm1), ("mixer", self.mixer))
         return (("norm1", self.norm1), ("mixer", self.mixer), ("norm2", self.norm2),
                 ("feed_forward", self.feed_forward))
 
@@ -45,6 +49,9 @@ class PreNormBlock:
         out: dict[str, TensorSpec] = {}
         for role, part in self._parts():
             out.update(part.expected_tensors(f"{prefix}{self.spec.name_of(role)}."))
+        if not self.has_feed_forward:
+            for name, spec in self.norm2.expected_tensors(f"{prefix}{self.spec.name_of('norm2')}.").items():
+                out[name] = replace(spec, optional=True)
         return out
 
     def bind(self, tensors, prefix, dtype, device) -> None:
@@ -66,18 +73,33 @@ class PreNormBlock:
                 warm(rows)
 
     def forward(self, residual: torch.Tensor, pending: Optional[torch.Tensor], batch, view,
-                writes: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+                writes: bool = True, plus: Optional[torch.Tensor] = None) -> tuple[torch.Tensor, torch.Tensor]:
+        """``plus``: float32 rows that join the stream in front of this layer (behind what is pending).  A first
+        norm that says ``takes_plus`` adds them in its own kernel; for any other they are added here."""
+        if plus is not None:
+            if getattr(self.norm1, "takes_plus", False):
+                x = self.norm1.forward(residual, pending, self.dtype, plus=plus)
+                return self._behind_first_norm(x, residual, batch, view, writes)
+            x = normalise(self.norm1, residual, pending, self.dtype)  # (the pending branch joins the stream)
+            residual.add_(plus)
+            pending = None
         if ((pending is None or isinstance(pending, Added)) and getattr(self.mixer, "takes_raw_rows", False)
                 and getattr(self.norm1, "folds_into_products", False) and RawRows.fits(residual, self.dtype)):
             # a few rows, the stream complete: the mixer's first product makes the norm itself (a kernel less)
             x = RawRows(residual, self.norm1, self.dtype)
         else:
             x = normalise(self.norm1, residual, pending, self.dtype)
+        return self._behind_first_norm(x, residual, batch, view, writes)
+
+    def _behind_first_norm(self, x, residual: torch.Tensor, batch, view, writes: bool):
         extra = {"residual": residual} if getattr(self.mixer, "adds_to_residual", False) else {}
-        if (extra and getattr(self.mixer, "folds_next_norm", False) and getattr(self.norm2, "folds_into_products", False)
+        if (extra and self.has_feed_forward and getattr(self.mixer, "folds_next_norm", False)
+                and getattr(self.norm2, "folds_into_products", False)
                 and getattr(self.feed_forward, "takes_scaled_rows", False)):
             extra["next_norm"] = self.norm2  # the norm between the two rides along with their products
         mixed = self.mixer.forward(x, batch, view, writes, **extra)
+        if not self.has_feed_forward:
+            return residual, mixed  # (the next norm adds it)
         x = normalise(self.norm2, residual, mixed, self.dtype)
         extra = {"residual": residual} if getattr(self.feed_forward, "adds_to_residual", False) else {}
         return residual, self.feed_forward.forward(x, **extra)

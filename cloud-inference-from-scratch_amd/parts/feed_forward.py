@@ -10,6 +10,7 @@ from typing import Optional
 
 import torch
 
+from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
 from .linear import linear
@@ -48,6 +49,45 @@ class GatedMLP(Part):
         return linear(linear(x, self.w_gate_up, epilogue="silu"), self.w_down, into=residual)
 
 
+class ClampedGatedMLP(Part):
+    """A dense gated feed-forward whose unit bounds its inputs: ``g = min(W_gate x, limit)``,
+    ``u = clamp(W_up x, -limit, limit)``, ``y = W_down (g * sigmoid(alpha g) * (u + offset))``.  ``limit``, ``alpha``
+    and ``offset`` are parameters (``limit=None``: unbounded; ``alpha=1, offset=0`` is ``silu(g) * u``); the unit is
+    computed in float32 from the product's rows."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: Optional[float] = None, alpha: float = 1.0,
+                 offset: float = 0.0, names: tuple[str, str, str] = ("gate", "up", "down")) -> None:
+        if min(hidden_size, intermediate_size) < 1 or (limit is not None and not limit > 0):
+            raise ValueError("sizes and the limit must be positive")
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.limit = float("inf") if limit is None else float(limit)
+        self.alpha, self.offset = float(alpha), float(offset)
+        self.names = tuple(names)
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        gate, up, down = self.names
+        return {
+            prefix + gate: TensorSpec((self.intermediate_size, self.hidden_size)),
+            prefix + up: TensorSpec((self.intermediate_size, self.hidden_size)),
+            prefix + down: TensorSpec((self.hidden_size, self.intermediate_size)),
+        }
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        gate, up, down = self.names
+        self.w_gate_up = torch.cat([tensors[prefix + gate], tensors[prefix + up]], dim=0).contiguous()
+        self.w_down = tensors[prefix + down].contiguous()
+
+    def warm_up(self, rows: int) -> None:
+        self.forward(torch.zeros((rows, self.hidden_size), dtype=self.w_down.dtype, device=self.w_down.device))
+
+    def forward(self, x, residual: Optional[torch.Tensor] = None):
+        hidden = ops.clamped_glu(linear(x, self.w_gate_up), self.limit, self.alpha, self.offset)
+        return linear(hidden, self.w_down)
+
+
 class NoFeedForward(Part):
     """A layer without a feed-forward: no tensors, and ``forward`` gives nothing to add."""
 
@@ -61,4 +101,5 @@ class NoFeedForward(Part):
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)
+register_part("feed_forward", "clamped_gated_mlp", ClampedGatedMLP)
 register_part("feed_forward", "none", NoFeedForward)

@@ -146,10 +146,14 @@ class StreamRows(Added):
 @dataclass
 class SummedBranch:
     """A branch output that is still a sum: ``main`` [T, H] (or ``None``) plus the ``P`` rows of each token in
-    ``parts`` (float32 [T, P, H]).  Whoever adds the branch sums them, in that order."""
+    ``parts`` (float32 [T, P, H]).  Whoever adds the branch sums them, in that order.  ``weights`` (float32 [T, P]):
+    each row of ``parts`` counts that much; ``main_gate`` (float32 [T], logits): ``main`` counts ``sigmoid`` of it.
+    Only a norm that applies them (``GroupedRMSNorm``) may be handed a branch that has them."""
 
     main: Optional[torch.Tensor]
     parts: Optional[torch.Tensor]
+    weights: Optional[torch.Tensor] = None
+    main_gate: Optional[torch.Tensor] = None
 
 
 @dataclass

@@ -53,6 +53,10 @@ class DecoderModel:
         # blocks that read what every earlier layer left (``keeps_history``) are handed a float32 tensor
         # [calls + 1, tokens, hidden] of the step: row 0 the embedding's rows, row i + 1 what call i left
         self.keeps_history = any(getattr(block, "keeps_history", False) for block in self.blocks)
+        # a run order that lets the embedding's rows join the stream again keeps a copy of them for the step
+        self.keeps_embedding = any(call.adds_embedding for call in spec.order)
+        if self.keeps_embedding and self.keeps_history:
+            raise ValueError("a run order adds the embedding's rows again to layers that average over the depth: not built")
         calls = [self.blocks[call.layer] for call in spec.order]
         if len(set(map(id, calls))) == len(calls):  # (a layer that runs twice has no single successor)
             for block, follower in zip(calls, calls[1:] + [None]):
@@ -138,9 +142,12 @@ class DecoderModel:
                              out=history[0] if history is not None else None, scale=self.spec.embedding_scale,
                              rows=rows)
         pending = StreamRows(rows) if rows is not None else None
+        embedded = residual.clone() if self.keeps_embedding else None
         for call in self.spec.order:
             block = self.blocks[call.layer]
             extra = {"history": history} if getattr(block, "keeps_history", False) else {}
+            if call.adds_embedding:
+                extra["plus"] = embedded
             residual, pending = block.forward(residual, pending, batch, cache.view(call.cache), call.writes, **extra)
         if batch.logit_rows.shape[0] == 0:  # a step of prompt portions that end before their prompts do
             return torch.empty((0, self.head.shape[0]), dtype=torch.float32, device=residual.device)

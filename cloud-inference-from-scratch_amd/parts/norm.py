@@ -109,9 +109,51 @@ class OnePlusRMSNorm(RMSNorm):
         """``residual += norm(branch)`` in float32; returns the new stream in ``out_dtype`` (if wanted).
         ``branch`` is a tensor or a ``SummedBranch``."""
         main, parts = (branch.main, branch.parts) if isinstance(branch, SummedBranch) else (branch, None)
+        if isinstance(branch, SummedBranch) and (branch.weights is not None or branch.main_gate is not None):
+            raise ValueError("this norm sums a branch's rows as they are: weights and gates are not its to apply")
         return ops.branch_norm_add(residual, main, self.weight, self.eps, out_dtype, parts=parts, want_rows=want_rows)
 
 
+class GroupedRMSNorm(Part):
+    """RMS norm whose statistics run over ``groups`` equal consecutive parts of the row: each part is divided by
+    its own ``sqrt(mean(part^2) + eps)``, and the whole row is multiplied by the weight.  One group is the plain RMS
+    norm.  The tensor is named like the norm itself (no ``.weight``).  The kernel that norms also adds whatever a
+    branch still owes the stream: a tensor, a ``SummedBranch`` (rows still to be summed, with weights per row where it
+    has them, and a gate on its main tensor), and ``plus`` (float32 rows that join the stream before the norm, such
+    as the embedding's rows once more).  Sums, statistics and scaling are float32."""
+
+    graph_safe = True
+    takes_plus = True
+
+    def __init__(self, size: int, eps: float, groups: int = 1) -> None:
+        if size <= 0 or not eps > 0 or groups < 1 or size % groups:
+            raise ValueError(f"a norm of {size} numbers in {groups} groups with eps {eps}: sizes positive, groups that divide")
+        if size + groups > ops.MAX_NORM_WIDTH:
+            raise ValueError(f"the norm kernels take rows of up to {ops.MAX_NORM_WIDTH} numbers, not {size}")
+        self.size, self.eps, self.groups = size, float(eps), groups
+        self.weight: Optional[torch.Tensor] = None
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        return {prefix.rstrip("."): TensorSpec((self.size,), init="norm", keeps_float32=True)}
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.weight = tensors[prefix.rstrip(".")].float().contiguous()
+        self.weight_f32 = self.weight
+
+    def forward(self, residual: torch.Tensor, branch, out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None, plus: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if isinstance(branch, (Added, RowSumsq)):
+            branch = None
+        extra = {}
+        if isinstance(branch, SummedBranch):
+            extra = dict(parts=branch.parts, part_weight=branch.weights, branch_gate=branch.main_gate)
+            branch = branch.main
+        return ops.group_norm_add(residual, branch, self.weight, self.groups, self.eps, out_dtype, rows=rows,
+                                  plus=plus, **extra)
+
+
 register_part("norm", "rms_norm", RMSNorm)
+register_part("norm", "rms_norm_groups", GroupedRMSNorm)
 register_part("norm", "rms_norm_one_plus", OnePlusRMSNorm)
 register_part("norm", "rms_norm_scalar", ScalarRMSNorm)

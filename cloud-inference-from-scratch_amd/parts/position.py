@@ -34,6 +34,7 @@ _TABLES: dict[tuple, tuple[torch.Tensor, torch.Tensor]] = {}
 class RotaryHalf(Part):
     graph_safe = True
     rotates = True
+    pairing = "halves"
 
     UNBOUNDED = 1 << 30   # what ``max_position`` reads as where the model names no longest position
     FIRST_ROWS = 4096     # the smallest table of a model without one
@@ -91,6 +92,15 @@ class RotaryHalf(Part):
         return kept
 
 
+class RotaryPairs(RotaryHalf):
+    """The same angles, with neighbours as partners: of the first ``rotary_dim`` numbers of a head, numbers
+    ``2i`` and ``2i + 1`` turn together by ``p * theta^(-2i / rotary_dim)``,
+    ``(u, v) -> (u cos - v sin, v cos + u sin)``.  The tables are those of the half-split pairing (an angle does
+    not know its partners); the kernel that turns the heads is told the pairing."""
+
+    pairing = "neighbours"
+
+
 class NoPosition(Part):
     graph_safe = True
     """Keys and queries enter the mixer as projected."""
@@ -111,4 +121,5 @@ class NoPosition(Part):
 
 
 register_part("position", "rotary_half", RotaryHalf)
+register_part("position", "rotary_pairs", RotaryPairs)
 register_part("position", "none", NoPosition)

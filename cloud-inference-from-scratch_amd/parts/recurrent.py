@@ -6,6 +6,9 @@
 (no weight), the heads are concatenated, multiplied by ``silu(W_g x)`` and projected.  The state ``S`` [heads, dim,
 vdim] is float32.
 
+``LightningAttention``: the same memory and read-out with activated queries, keys and values, no rotation, one
+norm with a weight over all heads' read-outs together and a ``sigmoid`` gate.
+
 ``GatedLinearRecurrence``: two branches of ``width`` channels, ``y = gelu_tanh(W_y x + b_y)`` and
 ``u = conv(W_x x + b_x)`` (a causal convolution over each channel's last ``taps`` inputs); per block of channels
 ``r = sigmoid(A_b u_b + a_b)``, ``i = sigmoid(B_b u_b + b_b)``; ``a = exp(-8 r softplus(lambda))``,
@@ -87,6 +90,81 @@ class Retention(Part):
         return linear(out, self.w_o)
 
 
+class LightningAttention(Part):
+    """Linear attention with a fixed decay per head and activated inputs: ``q = act(W_q x)``, ``k = act(W_k x)``
+    (heads x dim), ``v = act(W_v x)`` (heads x vdim), per head ``S_t = decay_h S_(t-1) + k_t v_t^T`` and
+    ``o_t = S_t^T q_t`` (no rotation, no other scale).  The heads' read-outs, concatenated, are divided by their
+    common root mean square and multiplied by the weight ``norm`` (one number per column), then by ``sigmoid(W_g x)``,
+    and projected.  The memory ``S`` [heads, dim, vdim] is float32, starts at zero and is carried in the request's
+    state slot; activations after the projection, decays, the walk and the norm are float32.  ``activation``,
+    ``norm_span`` (how many heads share a root mean square: all of them by default) and ``gate`` are parameters of
+    the kernels that ``Retention`` runs too."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, value_dim: int, decay: tuple, eps: float,
+                 activation: Optional[str] = "silu", gate: str = "sigmoid", norm_span: Optional[int] = None,
+                 norm_weight: bool = True) -> None:
+        for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("head_dim", head_dim),
+                            ("value_dim", value_dim)):
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be a positive integer, got {value!r}")
+        decay = tuple(float(d) for d in decay)
+        if len(decay) != num_heads:
+            raise ValueError(f"one decay per head: {len(decay)} for {num_heads} heads")
+        if not eps > 0:
+            raise ValueError("eps must be positive")
+        if activation not in ops.RETENTION_ACTIVATIONS or gate not in ops.RETENTION_GATES:
+            raise ValueError(f"activation {activation!r} or gate {gate!r} is none the kernels have")
+        ops.plan_retention(head_dim, value_dim)  # (refuses heads the kernel has no room for)
+        self.hidden_size, self.num_heads, self.head_dim, self.value_dim = hidden_size, num_heads, head_dim, value_dim
+        self.decay_values, self.eps = decay, float(eps)
+        self.activation, self.gate = activation, gate
+        self.norm_span = num_heads if norm_span is None else int(norm_span)
+        if self.norm_span < 1 or num_heads % self.norm_span:
+            raise ValueError(f"runs of {self.norm_span} heads do not divide {num_heads} heads")
+        self.has_norm_weight = bool(norm_weight)
+
+    def cache_need(self) -> FixedState:
+        return FixedState((self.num_heads, self.head_dim, self.value_dim))
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        h, d, v, hidden = self.num_heads, self.head_dim, self.value_dim, self.hidden_size
+        out = {
+            prefix + "q": TensorSpec((h * d, hidden)),
+            prefix + "k": TensorSpec((h * d, hidden)),
+            prefix + "v": TensorSpec((h * v, hidden)),
+            prefix + "g": TensorSpec((h * v, hidden)),
+            prefix + "o": TensorSpec((hidden, h * v)),
+        }
+        if self.has_norm_weight:
+            out[prefix + "norm"] = TensorSpec((h * v,), init="norm", keeps_float32=True)
+        return out
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.w_in = torch.cat([tensors[prefix + n] for n in ("q", "k", "v", "g")], dim=0).contiguous()
+        self.w_o = tensors[prefix + "o"].contiguous()
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=device)
+        self.norm_weight = tensors[prefix + "norm"].float().contiguous() if self.has_norm_weight else None
+
+    def warm_up(self, rows: int) -> None:
+        blank = lambda width: torch.zeros((rows, width), dtype=self.w_in.dtype, device=self.w_in.device)
+        linear(blank(self.hidden_size), self.w_in)
+        linear(blank(self.num_heads * self.value_dim), self.w_o)
+
+    def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+        if not writes:
+            raise ValueError("a recurrent mixer moves its state on whenever it runs")
+        h, d, v = self.num_heads, self.head_dim, self.value_dim
+        proj = linear(x, self.w_in)
+        out = ops.retention(proj, (0, h * d, 2 * h * d, 2 * h * d + h * v), None, None, 0, self.decay, view.state,
+                            batch.seq_slot, batch.positions, batch.q_start_loc, batch.sequences, h, d, v, self.eps,
+                            1.0, 0, activation=self.activation, norm_span=self.norm_span,
+                            norm_weight=self.norm_weight, gate=self.gate)
+        return linear(out, self.w_o)
+
+
 SCAN_SEGMENT_TOKENS = 64  # portions from which the recurrence's tokens are cut into stretches
 
 
@@ -148,4 +226,5 @@ class GatedLinearRecurrence(Part):
 
 
 register_part("mixer", "retention", Retention)
+register_part("mixer", "lightning_attention", LightningAttention)
 register_part("mixer", "gated_linear_recurrence", GatedLinearRecurrence)

@@ -7,7 +7,11 @@ the position in other ways.  Every step is a parameter of the part and may be le
   ``1 + coef * ln(floor((p + 1) / every) + 1)``);
 * ``score = q . k * scale``, then a smooth cap (``softcap``: ``c * tanh(score / c)``), then a bias on the distance
   itself (``slope_base = b``: head h of H loses ``2^(-b (h + 1) / H) * (i - j)``);
-* a window (``window``: the token itself and the ``window - 1`` before it);
+* a window (``window``: the token itself and the ``window - 1`` before it), or chunks (``chunk``: the token sees the
+  keys of its own chunk of that many positions up to itself; chunks are counted from position 0 of the sequence);
+* biases on the projections of queries, keys and values (``qkv_bias``);
+* a rotation of the first numbers of every query and key head by the position (``position``: a position part such
+  as ``rotary_pairs``, applied after the heads' norm);
 * a sink (``sink``: one learned number per head whose exponential stands in the softmax's denominator, and
   nowhere else);
 * a gate on every head's output (``head_gate``: ``sigmoid(W_g x)_h``, read from the layer's own input);
@@ -28,9 +32,11 @@ from typing import Optional
 import torch
 
 from ..cache.manager import PagedKV
+from ..config.specs import PartSpec
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
-from .base import Part, register_part
+from .base import Part, build_part, register_part
+from .latent_attention import positions_bound
 from .linear import linear
 
 _SAID_GENERIC: set = set()
@@ -47,7 +53,8 @@ class ScoredAttention(Part):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int,
                  scale: float, eps: float, window: Optional[int] = None, qk_norm: Optional[str] = None,
                  q_temperature: Optional[tuple] = None, softcap: Optional[float] = None,
-                 slope_base: Optional[float] = None, sink: bool = False, head_gate: bool = False) -> None:
+                 slope_base: Optional[float] = None, sink: bool = False, head_gate: bool = False,
+                 chunk: Optional[int] = None, qkv_bias: bool = False, position: Optional[PartSpec] = None) -> None:
         for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads),
                             ("head_dim", head_dim), ("value_dim", value_dim)):
             if isinstance(value, bool) or not isinstance(value, int) or value < 1:
@@ -58,6 +65,8 @@ class ScoredAttention(Part):
             raise ValueError(f"heads of up to 256 numbers, got {head_dim} and {value_dim}")
         if window is not None and window < 1:
             raise ValueError("window must be positive")
+        if chunk is not None and (isinstance(chunk, bool) or not isinstance(chunk, int) or chunk < 1 or window is not None):
+            raise ValueError(f"chunks hold a positive number of tokens and stand in a window's place, got {chunk!r}")
         if qk_norm not in ops.NORM_MODES:
             raise ValueError(f"qk_norm must be one of {list(ops.NORM_MODES)}, got {qk_norm!r}")
         if not eps > 0:
@@ -74,13 +83,18 @@ class ScoredAttention(Part):
         self.scale, self.eps, self.window = float(scale), float(eps), window
         self.qk_norm, self.q_temperature, self.softcap = qk_norm, q_temperature, softcap
         self.slope_base, self.sink, self.head_gate = slope_base, bool(sink), bool(head_gate)
+        self.chunk, self.qkv_bias = chunk, bool(qkv_bias)
+        self.position = build_part("position", position) if position is not None else None
+        if self.position is not None and self.position.rotates and self.position.rotary_dim > head_dim:
+            raise ValueError(f"{self.position.rotary_dim} turning numbers in heads of {head_dim}")
         # the head sizes the kernels and the cache see: those of the matrix-core form where it has them
         sizes = tuple(next((s for s in (64, 128) if s >= n), None) for n in (head_dim, value_dim))
         self.mfma_dims = sizes if sizes in ops.SCORED_MFMA_DIMS else None
         self.kernel_dim, self.kernel_vdim = self.mfma_dims or (_round8(head_dim), _round8(value_dim))
 
     def cache_need(self) -> PagedKV:
-        return PagedKV(self.num_kv_heads, self.kernel_dim, self.window,
+        # (a chunk's keys all lie inside a window of the chunk's length: pages behind it go back to the pool)
+        return PagedKV(self.num_kv_heads, self.kernel_dim, self.window if self.chunk is None else self.chunk,
                        value_dim=self.kernel_vdim if self.kernel_vdim != self.kernel_dim else None)
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
@@ -91,6 +105,10 @@ class ScoredAttention(Part):
             prefix + "v": TensorSpec((g * v, width)),
             prefix + "o": TensorSpec((width, h * v)),
         }
+        if self.qkv_bias:
+            out[prefix + "q.b"] = TensorSpec((h * d,))
+            out[prefix + "k.b"] = TensorSpec((g * d,))
+            out[prefix + "v.b"] = TensorSpec((g * v,))
         if self.qk_norm == "weight":
             out[prefix + "q.norm"] = TensorSpec((d,), init="norm", keeps_float32=True)
             out[prefix + "k.norm"] = TensorSpec((d,), init="norm", keeps_float32=True)
@@ -118,6 +136,10 @@ class ScoredAttention(Part):
             if h % 8:
                 blocks.append(pad(8 - h % 8))
         self.w_in = torch.cat(blocks, dim=0).contiguous()
+        self.b_in = None
+        if self.qkv_bias:
+            bias = torch.cat([tensors[prefix + "q.b"], tensors[prefix + "k.b"], tensors[prefix + "v.b"]], dim=0)
+            self.b_in = torch.cat([bias, bias.new_zeros(self.w_in.shape[0] - bias.shape[0])]).contiguous()
         self.q_weight = self.k_weight = None
         if self.qk_norm == "weight":
             self.q_weight = tensors[prefix + "q.norm"].float().contiguous()
@@ -136,22 +158,28 @@ class ScoredAttention(Part):
 
     def warm_up(self, rows: int) -> None:
         blank = lambda width: torch.zeros((rows, width), dtype=self.w_in.dtype, device=self.w_in.device)
-        linear(blank(self.hidden_size), self.w_in)
+        linear(blank(self.hidden_size), self.w_in, self.b_in)
         linear(blank(self.num_heads * self.kernel_vdim), self.w_o)
 
     def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
-        proj = linear(x, self.w_in)
+        proj = linear(x, self.w_in, self.b_in)
+        rotary = None
+        if self.position is not None and self.position.rotates:
+            if batch.max_context > self.position.max_position:
+                raise ValueError(f"position {batch.max_context - 1} is beyond the rotary table of {self.position.max_position}")
+            cos, sin = self.position.tables(x.device, positions_bound(batch))
+            rotary = (cos, sin, self.position.rotary_dim, getattr(self.position, "pairing", "halves") == "neighbours")
         q = ops.heads_prepare(proj, self.offsets, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim,
                               self.kernel_dim, self.kernel_vdim, self.qk_norm, self.q_weight, self.k_weight, self.eps,
                               self.q_temperature, batch.positions, batch.seq_of_token, batch.seq_slot,
-                              view.block_table, view.k_pool, view.v_pool, batch.tokens, write_kv=writes)
+                              view.block_table, view.k_pool, view.v_pool, batch.tokens, write_kv=writes, rotary=rotary)
         gate = proj[:, self.gate_offset:] if self.head_gate else None
         context = self.attend(q, gate, batch, view)
         return linear(context, self.w_o)
 
     def attend(self, q: torch.Tensor, gate, batch, view) -> torch.Tensor:
         shape = dict(window=self.window, scale=self.scale, softcap=self.softcap, slopes=self.slopes,
-                     sinks=self.sinks, gate=gate)
+                     sinks=self.sinks, gate=gate, chunk=self.chunk)
         h, g = self.num_heads, self.num_kv_heads
         group = h // g
         page_size = view.page_size
@@ -160,7 +188,8 @@ class ScoredAttention(Part):
             least = 1 if group <= 16 else 2 if group <= 32 else 4
             # the most keys a token sees in this step (a captured step: in any of its replays)
             bound = batch.static_plan.max_keys if batch.static_plan is not None else batch.max_context
-            bound = bound if self.window is None else min(bound, self.window)
+            reach = self.window if self.chunk is None else self.chunk  # the most keys a token sees, if bounded
+            bound = bound if reach is None else min(bound, reach)
 
             def shares(tiles: int, span: int) -> dict:
                 """Few tiles over many keys: the keys in shares of at least 128, about two workgroups a compute unit."""
