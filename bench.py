@@ -5,7 +5,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
                     [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 32768]
                     [--mixed-portions 16,64,248] [--other-shapes 7b,14b]
-    python bench.py --design polosun|givizen [--design-shapes 3b,7b] [--design-layers 12]
+    python bench.py --design polosun|givizen|nokipel [--design-shapes 3b,7b] [--design-layers 12]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -39,7 +39,12 @@ each with its share of the roofline of its own bytes and flops.  It prints one
 JSON line of its own.  ``--design givizen`` does the same for the Givizen design
 (window attention with shaped scores of two kinds in turn, each layer with
 routed experts and a shared one whose active sizes add up to the Qwen2.5
-shape's feed-forward).
+shape's feed-forward).  ``--design nokipel`` measures the Nokipel design (three
+layers of lightning attention to one of chunked softmax attention, dense
+bounded feed-forwards and routed experts in turn) beside the Givizen model of
+equal width, head sizes, expert sizes, vocabulary and layer count, the closest
+of the engine's models: the same attention and expert kernels with other
+options.
 """
 
 from __future__ import annotations
@@ -329,11 +334,87 @@ def givizen_costs(config, batch: int, context: float, tokens: int, elem: int) ->
     return moved, flops
 
 
+NOKIPEL_IDENTITY = 2
+NOKIPEL_GROUPS = (4, 2)
+
+
+def nokipel_raw(shape: dict, layers: int) -> dict:
+    """A Nokipel configuration with the width, vocabulary, head counts and head size of a Qwen2.5 shape: of every
+    four layers three have lightning attention (heads of 128 x 128, decays spread from 1 - 2^-5 to 1 - 2^-8) and one
+    has softmax attention in chunks of as many tokens as Givizen's shorter window, with a rotation over half of each
+    head; dense feed-forwards of the shape's size and routed ones take turns: 30 experts and 2 identity experts in 4
+    groups of which 2 are kept, 4 per token, experts and the shared one of Givizen's sizes; norms in 2 groups."""
+    width = shape["hidden_size"]
+    heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
+    dim = width // heads
+    expert_ff = shape["intermediate_size"] // (2 * GIVIZEN_TOP) // 64 * 64
+    shared_ff = shape["intermediate_size"] - GIVIZEN_TOP * expert_ff
+    dense = {"kind": "dense", "ff": shape["intermediate_size"], "limit": 7.0}
+    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff},
+              "router": {"experts": GIVIZEN_EXPERTS - NOKIPEL_IDENTITY, "identity": NOKIPEL_IDENTITY, "top": GIVIZEN_TOP,
+                         "scale": 2.0, "groups": {"count": NOKIPEL_GROUPS[0], "keep": NOKIPEL_GROUPS[1]}}}
+    memories = width // 128
+    lightning = {"heads": memories, "dim": 128, "vdim": 128,
+                 "decay": [1.0 - 2.0 ** (-5 - 3 * h / max(memories - 1, 1)) for h in range(memories)]}
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                 "mask": {"size": GIVIZEN_WINDOWS[0]}, "rot": {"base": 1000000.0, "dims": dim // 2}}
+    kinds = [
+        {"type": "lightning", "mixer": lightning, "mlp": dense},
+        {"type": "lightning", "mixer": lightning, "mlp": routed},
+        {"type": "lightning", "mixer": lightning, "mlp": dense},
+        {"type": "attention", "mixer": attention, "mlp": routed},
+    ]
+    return {"architecture": "Nokipel", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6, "groups": 2},
+            "embedding": {"scale": 1.0}, "layers": [kinds[i % 4] for i in range(layers)]}
+
+
+def nokipel_costs(config, batch: int, context: float, tokens: int, elem: int) -> tuple[float, float]:
+    """(bytes one decode step has to move, flops of a prefill of ``tokens`` tokens) for a Nokipel configuration
+    without a loop: every weight that a step touches once (of a layer's experts, the ones that ``batch`` tokens
+    choosing ``top`` of all router outputs at random are expected to hit; identity experts have none), each
+    request's keys and values inside the token's chunk, each lightning memory read and written in float32; products
+    at two flops per active weight and token, attention over the keys each token sees, the memories' updates and
+    read-outs."""
+    width, vocab = config.hidden_size, config.vocab_size
+    moved = float(vocab * width * elem)
+    flops = 2.0 * vocab * width
+    for layer in config.raw["layers"]:
+        m, mlp = layer["mixer"], layer["mlp"]
+        if layer["type"] == "lightning":
+            mixer = width * m["heads"] * (2 * m["dim"] + 3 * m["vdim"])
+            moved += batch * 2 * m["heads"] * m["dim"] * m["vdim"] * 4
+            flops += 2.0 * 2 * tokens * m["heads"] * m["dim"] * m["vdim"]
+        else:
+            mixer = width * (m["heads"] * m["dim"] + m["kv_heads"] * (m["dim"] + m["vdim"]) + m["heads"] * m["vdim"])
+            size = m["mask"]["size"] if m.get("mask") else None
+            seen = context if size is None else context % size + 1
+            moved += batch * seen * m["kv_heads"] * (m["dim"] + m["vdim"]) * elem
+            whole, rest = (tokens // size, tokens % size) if size else (0, tokens)
+            pairs = whole * size * (size + 1) / 2 + rest * (rest + 1) / 2
+            flops += 2.0 * pairs * m["heads"] * (m["dim"] + m["vdim"])
+        if mlp is None:
+            active = touched = 0.0
+        elif mlp["kind"] == "dense":
+            active = touched = 3.0 * width * mlp["ff"]
+        else:
+            router = mlp["router"]
+            experts, top = router["experts"], router["top"]
+            outputs = experts + router.get("identity", 0)
+            one = 3 * width * mlp["expert"]["ff"]
+            shared = 3 * width * mlp["shared"]["ff"] + width if mlp.get("shared") else 0
+            hit = experts * (1.0 - (1.0 - top / outputs) ** batch)
+            touched = width * outputs + shared + hit * one
+            active = width * outputs + shared + top * experts / outputs * one
+        moved += (mixer + touched) * elem
+        flops += 2.0 * tokens * (mixer + active)
+    return moved, flops
+
+
 def compare_designs(args) -> int:
-    """``--design polosun`` or ``--design givizen``: see the module's text."""
+    """``--design polosun``, ``--design givizen`` or ``--design nokipel``: see the module's text."""
     import torch
 
-    from cie_amd.config import GivizenConfig, PolosunConfig, Qwen2Config
+    from cie_amd.config import GivizenConfig, NokipelConfig, PolosunConfig, Qwen2Config
     from cie_amd.workloads import SHAPES
 
     elem = 2 if args.dtype == "bf16" else 4
@@ -341,11 +422,15 @@ def compare_designs(args) -> int:
     out = {}
     for name in [n for n in args.design_shapes.split(",") if n]:
         shape = SHAPES[name]
-        designs = {
-            args.design: (PolosunConfig.from_hf_config(polosun_raw(shape, layers)) if args.design == "polosun"
-                          else GivizenConfig.from_hf_config(givizen_raw(shape, layers))),
-            "qwen2": Qwen2Config.from_hf_config(dict(shape, num_hidden_layers=layers)),
-        }
+        if args.design == "nokipel":
+            designs = {"nokipel": NokipelConfig.from_hf_config(nokipel_raw(shape, layers)),
+                       "givizen": GivizenConfig.from_hf_config(givizen_raw(shape, layers))}
+        else:
+            designs = {
+                args.design: (PolosunConfig.from_hf_config(polosun_raw(shape, layers)) if args.design == "polosun"
+                              else GivizenConfig.from_hf_config(givizen_raw(shape, layers))),
+                "qwen2": Qwen2Config.from_hf_config(dict(shape, num_hidden_layers=layers)),
+            }
         out[name] = {}
         for design, config in designs.items():
             def costs(batch, context):
@@ -353,6 +438,8 @@ def compare_designs(args) -> int:
                     return polosun_costs(config, batch, context, args.prefill_tokens, elem)
                 if design == "givizen":
                     return givizen_costs(config, batch, context, args.prefill_tokens, elem)
+                if design == "nokipel":
+                    return nokipel_costs(config, batch, context, args.prefill_tokens, elem)
                 return (decode_bytes(config, layers, batch, context, elem), prefill_flops(config, layers, args.prefill_tokens))
 
             record = {}
@@ -376,15 +463,21 @@ def compare_designs(args) -> int:
                     "tokens_per_s": round(batch * steps / taken, 2), "ms_per_step": round(taken / steps * 1e3, 4),
                     "frac": round(costs(batch, mean_context)[0] / (taken / steps) / 1e9 / HBM_GBPS, 4)}
             out[name][design] = record
+    givizen_layers = (f"attention (window {GIVIZEN_WINDOWS[0]}) and attention_2 (window {GIVIZEN_WINDOWS[1]}) in turn, each "
+                      f"with {GIVIZEN_EXPERTS} experts, {GIVIZEN_TOP} per token, and a shared expert")
+    beside = ("the Givizen model of equal width, head and expert sizes" if args.design == "nokipel"
+              else "the Qwen2.5 decoder of equal width, feed-forward")
     print(json.dumps({
-        "metric": f"{args.design.capitalize()} beside the Qwen2.5 decoder of equal width, feed-forward, vocabulary and {layers} layers",
+        "metric": f"{args.design.capitalize()} beside {beside}, vocabulary and {layers} layers",
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": args.dtype,
         "data": "synthetic (seeded uniform-random token ids, random weights N(0, 0.02))",
         "config": {"layers": layers, "context": args.context, "prefill_tokens": args.prefill_tokens, "page_size": PAGE,
                    "design_layers": ("retention, latent_attention, rglru in turn, each with a dense feed-forward"
-                                     if args.design == "polosun" else
-                                     f"attention (window {GIVIZEN_WINDOWS[0]}) and attention_2 (window {GIVIZEN_WINDOWS[1]}) in turn, each "
-                                     f"with {GIVIZEN_EXPERTS} experts, {GIVIZEN_TOP} per token, and a shared expert")},
+                                     if args.design == "polosun" else givizen_layers if args.design == "givizen" else
+                                     f"lightning + dense, lightning + experts, lightning + dense, attention (chunks of "
+                                     f"{GIVIZEN_WINDOWS[0]}) + experts in turn; {GIVIZEN_EXPERTS - NOKIPEL_IDENTITY} experts and "
+                                     f"{NOKIPEL_IDENTITY} identity experts in {NOKIPEL_GROUPS[0]} groups ({NOKIPEL_GROUPS[1]} kept), "
+                                     f"{GIVIZEN_TOP} per token, and a gated shared expert; beside it Givizen: " + givizen_layers)},
         "shapes": out,
     }))
     return 0
@@ -411,8 +504,9 @@ def main(argv=None) -> int:
                              "(default 16,64,248; '' for none, as with --no-points)")
     parser.add_argument("--other-shapes", default="7b,14b",
                         help="further shapes whose decode at the main batch and context and whose prefill go into the points ('' for none)")
-    parser.add_argument("--design", default=None, choices=["polosun", "givizen"],
-                        help="instead of the default record: this design beside the Qwen2.5 decoder of equal size")
+    parser.add_argument("--design", default=None, choices=["polosun", "givizen", "nokipel"],
+                        help="instead of the default record: this design beside the Qwen2.5 decoder of equal size "
+                             "(nokipel: beside the Givizen model of equal size)")
     parser.add_argument("--design-shapes", default="3b,7b", help="the Qwen2.5 shapes whose sizes the comparison takes")
     parser.add_argument("--design-layers", type=int, default=12, help="layers of both models in the comparison")
     args = parser.parse_args(argv)
