@@ -212,7 +212,8 @@ CIE_API int cie_branch_norm_add(void* stream, int bdtype, int dtype, float* resi
 // The residual add of a layer that norms what its sublayers read, with everything a branch can still owe the stream,
 // and an RMS norm whose statistics run over equal consecutive parts of the row:
 //
-//   x = residual[row] + branch[row] * sigmoid(branch_gate[row])            (branch; the gate one logit per row)
+//   x = residual[row] + branch[row] * sigmoid(branch_gate[row])            (branch; the gate one logit per row, rows
+//                                                                           `gate_stride` floats apart)
 //                     + sum_p part_weight[row, p] * parts[row, p, :]       (float32 rows still to be summed, in order)
 //                     + plus[row]                                          (float32 rows, e.g. the embedding's again)
 //   y[g] = x[g] / sqrt(mean(x[g]^2) + eps) * weight[g]                     for each of the `groups` parts g of the row
@@ -222,8 +223,8 @@ CIE_API int cie_branch_norm_add(void* stream, int bdtype, int dtype, float* resi
 // statistics need no barrier per group.
 template <typename B, typename T>
 __global__ void group_norm_add_kernel(float* __restrict__ residual, const B* __restrict__ branch,
-                                      const float* __restrict__ branch_gate, const float* __restrict__ parts,
-                                      const float* __restrict__ part_weight, int n_parts,
+                                      const float* __restrict__ branch_gate, int gate_stride,
+                                      const float* __restrict__ parts, const float* __restrict__ part_weight, int n_parts,
                                       const float* __restrict__ plus, const float* __restrict__ weight,
                                       T* __restrict__ out, const int* __restrict__ rows, int hidden, int groups,
                                       float eps, int write_residual) {
@@ -233,7 +234,7 @@ __global__ void group_norm_add_kernel(float* __restrict__ residual, const B* __r
     const size_t row = rows ? rows[out_row] : out_row;
     float* res = residual + row * hidden;
     const B* add = branch ? branch + row * hidden : nullptr;
-    const float open = (branch && branch_gate) ? 1.0f / (1.0f + expf(-branch_gate[row])) : 1.0f;
+    const float open = (branch && branch_gate) ? 1.0f / (1.0f + expf(-branch_gate[row * gate_stride])) : 1.0f;
     const float* extra = n_parts > 0 ? parts + row * n_parts * hidden : nullptr;
     const float* extra_w = (n_parts > 0 && part_weight) ? part_weight + row * n_parts : nullptr;
     const float* more = plus ? plus + row * hidden : nullptr;
@@ -267,10 +268,10 @@ __global__ void group_norm_add_kernel(float* __restrict__ residual, const B* __r
 
 // bdtype: storage type of `branch` (ignored without one); dtype: type of `out`.  `weight` float32 [hidden].
 CIE_API int cie_group_norm_add(void* stream, int bdtype, int dtype, float* residual, const void* branch,
-                               const float* branch_gate, const float* parts, const float* part_weight, int n_parts,
-                               const float* plus, const float* weight, void* out, const int* rows, int n_rows,
+                               const float* branch_gate, int gate_stride, const float* parts, const float* part_weight,
+                               int n_parts, const float* plus, const float* weight, void* out, const int* rows, int n_rows,
                                int hidden, int groups, float eps) {
-    if (n_rows < 0 || hidden <= 0 || groups <= 0 || hidden % groups || !(eps > 0.f) || n_parts < 0 ||
+    if (n_rows < 0 || hidden <= 0 || groups <= 0 || hidden % groups || !(eps > 0.f) || n_parts < 0 || gate_stride < 1 ||
         (n_parts > 0 && !parts) || (static_cast<size_t>(hidden) + groups) * sizeof(float) > 64 * 1024 || !weight || !out)
         return CIE_BAD_ARGUMENT;
     if (n_rows == 0) return CIE_OK;
@@ -281,15 +282,18 @@ CIE_API int cie_group_norm_add(void* stream, int bdtype, int dtype, float* resid
     const int write_residual = (rows == nullptr && (branch || n_parts > 0 || plus)) ? 1 : 0;
     if (dtype == CIE_F32 && (bdtype == CIE_F32 || !branch))
         group_norm_add_kernel<float, float><<<n_rows, threads, lds, s>>>(
-            residual, static_cast<const float*>(branch), branch_gate, parts, part_weight, n_parts, plus, weight,
+            residual, static_cast<const float*>(branch), branch_gate, gate_stride, parts, part_weight, n_parts, plus,
+            weight,
             static_cast<float*>(out), rows, hidden, groups, eps, write_residual);
     else if (dtype == CIE_BF16 && (bdtype == CIE_BF16 || !branch))
         group_norm_add_kernel<bf16_t, bf16_t><<<n_rows, threads, lds, s>>>(
-            residual, static_cast<const bf16_t*>(branch), branch_gate, parts, part_weight, n_parts, plus, weight,
+            residual, static_cast<const bf16_t*>(branch), branch_gate, gate_stride, parts, part_weight, n_parts, plus,
+            weight,
             static_cast<bf16_t*>(out), rows, hidden, groups, eps, write_residual);
     else if (dtype == CIE_BF16 && bdtype == CIE_F32)
         group_norm_add_kernel<float, bf16_t><<<n_rows, threads, lds, s>>>(
-            residual, static_cast<const float*>(branch), branch_gate, parts, part_weight, n_parts, plus, weight,
+            residual, static_cast<const float*>(branch), branch_gate, gate_stride, parts, part_weight, n_parts, plus,
+            weight,
             static_cast<bf16_t*>(out), rows, hidden, groups, eps, write_residual);
     else
         return CIE_BAD_ARGUMENT;

@@ -50,7 +50,8 @@ retention_turn_kernel(const T* __restrict__ proj, long ldp, int q_off, int k_off
     const int half = rot / 2;
     const T* row = proj + static_cast<size_t>(token) * ldp;
     const size_t at = static_cast<size_t>(positions[token]) * half;
-    for (int idx = threadIdx.x; idx < heads * padded; idx += blockDim.x) {
+    // (few tokens: the workgroups of a token, blockIdx.y, share its heads' numbers)
+    for (int idx = blockIdx.y * blockDim.x + threadIdx.x; idx < heads * padded; idx += blockDim.x * gridDim.y) {
         const int head = idx / padded;
         const int d = idx - head * padded;
         float qv = 0.f, kv = 0.f;
@@ -251,6 +252,44 @@ retention_norm_kernel(float* __restrict__ raw, long plane, int parts, const T* _
     }
 }
 
+// The same for runs wider than a wave takes well (a norm over all heads of a token): one workgroup per (token, run),
+// the summed columns wait in LDS, the waves' sums of squares meet there in the waves' order.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+retention_norm_wide_kernel(const float* __restrict__ raw, long plane, int parts, const T* __restrict__ proj, long ldp,
+                           int g_off, T* __restrict__ out, int heads, int vdim, float eps, int span,
+                           const float* __restrict__ weight, int gate_act) {
+    extern __shared__ float wide[];  // [span * vdim] the run's columns, then one sum of squares per wave
+    const int runs = heads / span;
+    const int token = blockIdx.x / runs;
+    const int first = (blockIdx.x - token * runs) * span * vdim;
+    const int width = span * vdim;
+    float* partial = wide + width;
+    const float* o = raw + static_cast<size_t>(token) * heads * vdim + first;
+    float sum_sq = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float v = o[c];
+        for (int p = 1; p < parts; ++p) v += o[static_cast<size_t>(p) * plane + c];  // (the parts in their order)
+        wide[c] = v;  // (this thread's own column: it reads it again below)
+        sum_sq += v * v;
+    }
+    sum_sq = wave_sum(sum_sq);
+    if (threadIdx.x % kWave == 0) partial[threadIdx.x / kWave] = sum_sq;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < static_cast<int>(blockDim.x) / kWave; ++w) total += partial[w];
+    const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+    const T* gate = proj + static_cast<size_t>(token) * ldp + g_off + first;
+    T* dst = out + static_cast<size_t>(token) * heads * vdim + first;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const float g = to_float(gate[c]);
+        const float open = gate_act == 1 ? sigmoidf(g) : g * sigmoidf(g);
+        float y = wide[c] * inv;
+        if (weight) y *= weight[first + c];
+        dst[c] = from_float<T>(y * open);
+    }
+}
+
 template <typename T, int DS>
 int launch_retention(hipStream_t s, dim3 grid, int threads, size_t lds, const void* proj, long ldp, int v_off,
                      const float* turned, const float* decay, float* state, const int* seq_slot, const int* q_start_loc,
@@ -397,11 +436,15 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
         return CIE_BAD_ARGUMENT;
     if (sequences == 0 || tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    // a step of few tokens: up to sixteen workgroups a token, so that a single token's heads do not wait for one
+    const int turn_blocks = (heads * padded + 255) / 256;
+    const int per_token = tokens >= 256 ? 1 : (turn_blocks < 16 ? turn_blocks : 16);
+    const dim3 turn_grid(tokens, per_token);
     if (dtype == CIE_F32)
-        retention_turn_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(proj), ldp, q_off, k_off, cos_table,
+        retention_turn_kernel<float><<<turn_grid, 256, 0, s>>>(static_cast<const float*>(proj), ldp, q_off, k_off, cos_table,
                                                            sin_table, rot, positions, turned, heads, dim, padded, key_scale, act);
     else if (dtype == CIE_BF16)
-        retention_turn_kernel<bf16_t><<<tokens, 256, 0, s>>>(static_cast<const bf16_t*>(proj), ldp, q_off, k_off, cos_table,
+        retention_turn_kernel<bf16_t><<<turn_grid, 256, 0, s>>>(static_cast<const bf16_t*>(proj), ldp, q_off, k_off, cos_table,
                                                             sin_table, rot, positions, turned, heads, dim, padded, key_scale, act);
     else
         return CIE_BAD_ARGUMENT;
@@ -425,6 +468,21 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
 #undef CIE_RETENTION
     if (code != CIE_OK) return code;
     const int items = tokens * (heads / norm_span);
+    const int width = norm_span * vdim;
+    if (width > 256 && (static_cast<size_t>(width) + 16) * sizeof(float) <= 60 * 1024) {
+        // (which kernel norms depends on the run's width alone, never on what else the step holds)
+        const int threads = width >= 2048 ? 1024 : width >= 1024 ? 512 : 256;
+        const size_t norm_lds = (static_cast<size_t>(width) + 16) * sizeof(float);
+        if (dtype == CIE_F32)
+            retention_norm_wide_kernel<float><<<items, threads, norm_lds, s>>>(
+                raw, plane, parts, static_cast<const float*>(proj), ldp, g_off, static_cast<float*>(out), heads, vdim, eps,
+                norm_span, norm_weight, gate_act);
+        else
+            retention_norm_wide_kernel<bf16_t><<<items, threads, norm_lds, s>>>(
+                raw, plane, parts, static_cast<const bf16_t*>(proj), ldp, g_off, static_cast<bf16_t*>(out), heads, vdim,
+                eps, norm_span, norm_weight, gate_act);
+        return cie_after_launch();
+    }
     const int blocks = (items + 3) / 4;
     if (dtype == CIE_F32)
         retention_norm_kernel<float><<<blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const float*>(proj), ldp, g_off,

@@ -1126,7 +1126,7 @@ def group_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weigh
     """``residual += branch * sigmoid(branch_gate) + sum_p part_weight[:, p] * parts[:, p] + plus`` (whatever of it
     is given; float32, in place unless ``rows``), then the RMS norm of every row in ``groups`` equal consecutive
     parts, each over its own root mean square, the whole times ``weight`` (float32 [H]).  ``branch`` [T, H] float32
-    or ``out_dtype``; ``branch_gate`` float32 [T] (logits); ``parts`` float32 [T, P, H]; ``part_weight`` float32
+    or ``out_dtype``; ``branch_gate`` float32 [T] (logits; any stride); ``parts`` float32 [T, P, H]; ``part_weight`` float32
     [T, P]; ``plus`` float32 [T, H].  With ``rows`` (int32 [n]) only those rows come back, in that order."""
     _gpu("residual", residual, torch.float32, 2)
     tokens, hidden = residual.shape
@@ -1139,10 +1139,14 @@ def group_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weigh
         _gpu("branch", branch, dims=2)
         if not (branch.shape == residual.shape and branch.dtype in (torch.float32, out_dtype)):
             raise ValueError(f"branch {tuple(branch.shape)} {branch.dtype} does not fit {tuple(residual.shape)} {out_dtype}")
+    gate_stride = 1
     if branch_gate is not None:
-        _gpu("branch_gate", branch_gate, torch.float32, 1)
+        # (one logit per row; the rows may lie apart, as the first column of a wider product's result does)
+        if not (branch_gate.is_cuda and branch_gate.dtype == torch.float32 and branch_gate.dim() == 1):
+            raise ValueError("branch_gate must be a float32 GPU vector")
         if branch is None or branch_gate.shape[0] != tokens:
             raise ValueError("a gate comes with a branch, one logit per row")
+        gate_stride = max(branch_gate.stride(0), 1)
     n_parts = 0
     if parts is not None:
         _gpu("parts", parts, torch.float32, 3)
@@ -1164,7 +1168,7 @@ def group_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weigh
     out = torch.empty((n_out, hidden), dtype=out_dtype, device=residual.device)
     _run("cie_group_norm_add", load_library().cie_group_norm_add(
         _stream(), _i(_code(branch.dtype if branch is not None else out_dtype)), _i(_code(out_dtype)), _ptr(residual),
-        _ptr(branch), _ptr(branch_gate), _ptr(parts), _ptr(part_weight), _i(n_parts), _ptr(plus), _ptr(weight),
+        _ptr(branch), _ptr(branch_gate), _i(gate_stride), _ptr(parts), _ptr(part_weight), _i(n_parts), _ptr(plus), _ptr(weight),
         _ptr(out), _ptr(rows), _i(n_out), _i(hidden), _i(groups), _f(eps)))
     return out
 

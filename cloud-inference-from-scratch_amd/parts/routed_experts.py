@@ -141,7 +141,7 @@ class RoutedExperts(Part):
             hidden = ops.clamped_glu(linear(x, self.w_shared_gate_up), self.shared_limit, self.alpha, self.offset)
             shared = linear(hidden, self.w_shared_down)
             if self.w_shared_gate is not None:
-                gate = linear(x, self.w_shared_gate, out_dtype=torch.float32)[:, 0].contiguous()
+                gate = linear(x, self.w_shared_gate, out_dtype=torch.float32)[:, 0]  # (the norm kernel strides over the rows)
         weights = None if on_input else route.pair_weight.view(tokens, self.top)
         return SummedBranch(shared, parts, weights=weights, main_gate=gate)
 

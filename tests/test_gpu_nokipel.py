@@ -78,6 +78,11 @@ MECHANISMS = {
                             "mixer": {"heads": 3, "dim": 40, "vdim": 8, "decay": [0.5, 0.9, 0.999]}},
     "lightning_heads_of_64": {"type": "lightning", "mlp": None,
                               "mixer": {"heads": 2, "dim": 64, "vdim": 64, "decay": [0.75, 0.998046875]}},
+    # rows of all heads' read-outs wider than one wave norms: 1,080 and 2,176 numbers
+    "lightning_wide_rows": {"type": "lightning", "mlp": None,
+                            "mixer": {"heads": 9, "dim": 4, "vdim": 120, "decay": [0.5 + 0.055 * h for h in range(9)]}},
+    "lightning_many_heads": {"type": "lightning", "mlp": None,
+                             "mixer": {"heads": 17, "dim": 8, "vdim": 128, "decay": [1.0 - 2.0 ** -(1 + h % 9) for h in range(17)]}},
     "dense": {"type": "lightning", "mixer": TINY_MIXER, "mlp": {"kind": "dense", "ff": 44, "limit": 0.5}},
     "dense_wide_limit": {"type": "lightning", "mixer": TINY_MIXER, "mlp": {"kind": "dense", "ff": 20, "limit": 30.0}},
     "experts": {"type": "lightning", "mixer": TINY_MIXER, "mlp": MOE_FULL},
@@ -426,6 +431,8 @@ def test_the_norm_in_groups_adds_what_the_stream_is_owed(dtype):
         part_weight = torch.rand(rows, max(n_parts, 1), generator=g) * 2
         plus = torch.randn(rows, hidden, generator=g)
         weight = 1.0 + 0.3 * torch.randn(hidden, generator=g)
+        wide_gate = torch.zeros(rows, 5).cuda()
+        wide_gate[:, 2] = gate.cuda()       # (one logit per row, the rows five floats apart)
         tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=1e-2, rtol=1e-2)
         for use_branch, use_gate, use_parts, use_weight, use_plus in (
                 (True, True, True, True, True), (True, False, False, False, False), (False, False, True, True, False),
@@ -435,7 +442,7 @@ def test_the_norm_in_groups_adds_what_the_stream_is_owed(dtype):
             stream = residual.clone().cuda()
             out = ops.group_norm_add(
                 stream, branch.cuda() if use_branch else None, weight.cuda(), groups, 1e-5, dtype,
-                branch_gate=gate.cuda() if use_gate else None, parts=parts.cuda() if use_parts else None,
+                branch_gate=wide_gate[:, 2] if use_gate else None, parts=parts.cuda() if use_parts else None,
                 part_weight=part_weight.cuda() if use_weight else None, plus=plus.cuda() if use_plus else None)
             want = residual.double()
             if use_branch:
