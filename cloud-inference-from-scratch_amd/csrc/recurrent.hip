@@ -217,6 +217,198 @@ retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* _
 }
 #undef CIE_RETENTION_FETCH
 
+// (b') The same walk for sequences that bring many tokens (a prompt's portion), in blocks of 32 tokens on the matrix
+// cores, float32 throughout (`v_mfma_f32_16x16x4_f32`: operands and sums are plain float32).  With S the memory in
+// front of a block, i and j tokens of the block and f the head's decay:
+//     o_i   = f^(i+1) * (S^T q_i)  +  sum_{j <= i} f^(i-j) (q_i . k_j) v_j
+//     S_new = f^n * S  +  sum_j f^(n-1-j) k_j v_j^T          (n the block's tokens: 32, or fewer at the end)
+// One workgroup of four waves takes (sequence, head, 16 value columns) and walks the blocks in order.  The block's
+// queries, keys and values wait in LDS (fetched into registers a block ahead).  Wave w keeps rows of S in the matrix
+// cores' result layout, where they serve as the second operand of S^T q as they are; it makes one 16 x 16 tile of
+// q . k (the tile above the diagonal is zero), and its share of S^T q, of the block's own sum (tokens 8w .. 8w + 7)
+// and of the new S; the waves' shares of o meet in LDS in the waves' order.  Powers of f come from a table made by
+// repeated multiplication, as the walk token by token makes them.
+typedef float acc4_t __attribute__((ext_vector_type(4)));
+constexpr int kBlockTokens = 32;
+constexpr int kBlockCols = 16;
+constexpr int kScoreStride = kBlockTokens + 4;
+
+// TPW: tiles of 16 rows of S that a wave keeps (the head's `padded` numbers are at most 64 * TPW)
+template <typename T, int TPW>
+__global__ void __launch_bounds__(256)
+retention_blocks_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* __restrict__ turned,
+                        const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ seq_slot,
+                        const int* __restrict__ q_start_loc, float* __restrict__ raw, int heads, int dim, int vdim,
+                        int padded, int act) {
+    extern __shared__ float4 lds4[];
+    float* lds = reinterpret_cast<float*>(lds4);
+    const int stride = padded + 4;                       // (a row's start moves on by four banks)
+    float* q_s = lds;                                    // [32][stride]
+    float* k_s = q_s + kBlockTokens * stride;            // [32][stride]
+    float* v_s = k_s + kBlockTokens * stride;            // [32][16]
+    float* p_s = v_s + kBlockTokens * kBlockCols;        // [32][36]: f^(i-j) (q_i . k_j), zero above the diagonal
+    float* red = p_s + kBlockTokens * kScoreStride;      // [4][32][16]: the waves' shares of o
+    float* pw = red + 4 * kBlockTokens * kBlockCols;     // [33]: powers of the decay
+    const int seq = blockIdx.x / heads;
+    const int head = blockIdx.x - seq * heads;
+    const int v0 = blockIdx.y * kBlockCols;
+    const int first = q_start_loc[seq];
+    const int count = q_start_loc[seq + 1] - first;
+    const int slot = seq_slot[seq];
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int l16 = lane % 16;
+    const int g = lane / 16;
+    const int tiles = padded / 16;
+    const bool col_ok = v0 + l16 < vdim;
+    if (threadIdx.x == 0) {
+        float f = 1.0f;
+        const float fade = decay[head];
+        for (int n = 0; n <= kBlockTokens; ++n) {
+            pw[n] = f;
+            f *= fade;
+        }
+    }
+    // rows of S: lane (g, l16), number r of tile t holds row 16 t + 4 r + g of column v0 + l16
+    float* mem = state + ((static_cast<size_t>(slot) * heads + head) * dim) * vdim + v0 + l16;
+    acc4_t S[TPW];
+#pragma unroll
+    for (int u = 0; u < TPW; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 16 * (wave * TPW + u) + 4 * r + g;
+            S[u][r] = (col_ok && row < dim) ? mem[static_cast<size_t>(row) * vdim] : 0.f;
+        }
+    const int pieces = padded / 2;                       // 16-byte pieces of one token's query and key
+    piece_t ahead[4 * TPW];
+    float ahead_v[2];
+#define CIE_BLOCKS_FETCH(from)                                                                                        \
+    {                                                                                                                 \
+        const int fetch_n = min(kBlockTokens, count - (from));                                                        \
+        _Pragma("unroll") for (int i = 0; i < 4 * TPW; ++i) {                                                         \
+            const int idx = min(static_cast<int>(threadIdx.x) + i * 256, fetch_n * pieces - 1);                       \
+            const int t = idx / pieces;                                                                               \
+            ahead[i] = *reinterpret_cast<const piece_t*>(                                                             \
+                turned + (static_cast<size_t>(first + (from) + t) * heads + head) * 2 * padded + (idx - t * pieces) * 4); \
+        }                                                                                                             \
+        _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                               \
+            const int idx = static_cast<int>(threadIdx.x) + i * 256;                                                  \
+            const int t = min(idx / kBlockCols, fetch_n - 1);                                                         \
+            const int c = min(v0 + idx % kBlockCols, vdim - 1);                                                       \
+            ahead_v[i] = activated(                                                                                   \
+                to_float(proj[static_cast<size_t>(first + (from) + t) * ldp + v_off + head * vdim + c]), act);        \
+        }                                                                                                             \
+    }
+    if (count > 0) CIE_BLOCKS_FETCH(0)
+    for (int c0 = 0; c0 < count; c0 += kBlockTokens) {
+        const int cn = min(kBlockTokens, count - c0);
+        // the block into LDS; rows past the block's last token are zero
+#pragma unroll
+        for (int i = 0; i < 4 * TPW; ++i) {
+            const int idx = threadIdx.x + i * 256;
+            if (idx < kBlockTokens * pieces) {
+                const int t = idx / pieces;
+                const int within = idx - t * pieces;
+                const int side = within / (padded / 4);  // 0: the query, 1: the key
+                const piece_t value = t < cn ? ahead[i] : piece_t{0.f, 0.f, 0.f, 0.f};
+                *reinterpret_cast<piece_t*>((side ? k_s : q_s) + t * stride + (within - side * (padded / 4)) * 4) = value;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = threadIdx.x + i * 256;
+            const int t = idx / kBlockCols;
+            v_s[idx] = (t < cn && v0 + idx % kBlockCols < vdim) ? ahead_v[i] : 0.f;
+        }
+        __syncthreads();
+        if (c0 + kBlockTokens < count) CIE_BLOCKS_FETCH(c0 + kBlockTokens)
+        // this wave's tile of the scores
+        {
+            const int ti = wave >> 1, tj = wave & 1;
+            acc4_t p = {0.f, 0.f, 0.f, 0.f};
+            if (tj <= ti) {
+                const float* qa = q_s + (16 * ti + l16) * stride + g;
+                const float* kb = k_s + (16 * tj + l16) * stride + g;
+                for (int kk = 0; kk < padded / 4; ++kk)
+                    p = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[4 * kk], kb[4 * kk], p, 0, 0, 0);
+            }
+            const int j = 16 * tj + l16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 16 * ti + 4 * g + r;
+                p_s[i * kScoreStride + j] = j <= i ? p[r] * pw[i - j] : 0.f;
+            }
+        }
+        // this wave's share of S^T q, faded by the tokens' places in the block
+        acc4_t o[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) {
+            const int t = wave * TPW + u;
+            if (t < tiles) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int d = 16 * t + 4 * r + g;
+                    o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(q_s[l16 * stride + d], S[u][r], o[0], 0, 0, 0);
+                    o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(q_s[(16 + l16) * stride + d], S[u][r], o[1], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[rt][r] *= pw[16 * rt + 4 * g + r + 1];
+        __syncthreads();
+        // ... of the block's own sum: tokens 8 w .. 8 w + 7
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            const int j = 8 * wave + 4 * kk + g;
+            const float vb = v_s[j * kBlockCols + l16];
+            o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[l16 * kScoreStride + j], vb, o[0], 0, 0, 0);
+            o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[(16 + l16) * kScoreStride + j], vb, o[1], 0, 0, 0);
+        }
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                red[(wave * kBlockTokens + 16 * rt + 4 * g + r) * kBlockCols + l16] = o[rt][r];
+        // ... and of the new S
+        {
+            const float keep = pw[cn];
+            const int mine = 4 * (l16 % 4) + l16 / 4;    // the row of a tile that stands at place l16 of the layout
+#pragma unroll
+            for (int u = 0; u < TPW; ++u) {
+                const int t = wave * TPW + u;
+                if (t < tiles) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) S[u][r] *= keep;
+#pragma unroll
+                    for (int kk = 0; kk < kBlockTokens / 4; ++kk) {
+                        const int j = 4 * kk + g;
+                        const float ka = k_s[j * stride + 16 * t + mine] * pw[max(cn - 1 - j, 0)];
+                        S[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka, v_s[j * kBlockCols + l16], S[u], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < cn * kBlockCols; idx += blockDim.x) {
+            const int c = idx % kBlockCols;
+            if (v0 + c >= vdim) continue;
+            float sum = red[idx];
+            for (int w = 1; w < 4; ++w) sum += red[w * kBlockTokens * kBlockCols + idx];
+            raw[static_cast<size_t>(first + c0 + idx / kBlockCols) * heads * vdim + head * vdim + v0 + c] = sum;
+        }
+    }
+#undef CIE_BLOCKS_FETCH
+#pragma unroll
+    for (int u = 0; u < TPW; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 16 * (wave * TPW + u) + 4 * r + g;
+            if (col_ok && row < dim) mem[static_cast<size_t>(row) * vdim] = S[u][r];
+        }
+}
+
 // o / sqrt(mean(o^2) + eps) [* weight] * gate: one wave per (token, run of `span` heads).  The mean runs over the
 // `span` heads of a run together (1: every head by itself; `heads`: all of a token's heads as one vector); `weight`
 // [heads * vdim] float32 or null; the gate is silu(g) (gate_act 0) or sigmoid(g) (1) of the projection's gate columns.
@@ -417,8 +609,16 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
                           const int* seq_slot, const int* positions, const int* q_start_loc, float* turned, float* raw,
                           void* out, int tokens, int sequences, int heads, int dim, int vdim, int rows_per_thread,
                           int groups, int parts, int slice, int chunk, float eps, float key_scale, int act,
-                          int norm_span, const float* norm_weight, int gate_act) {
+                          int norm_span, const float* norm_weight, int gate_act, int blocks) {
     if (act < 0 || act > 1 || norm_span < 1 || heads % norm_span || gate_act < 0 || gate_act > 1) return CIE_BAD_ARGUMENT;
+    if (blocks) {
+        // the walk in blocks on the matrix cores: one plane of o, queries and keys padded to whole tiles of 16
+        groups = 1;
+        rows_per_thread = 16;
+        parts = (dim + 15) / 16;
+        slice = vdim < kBlockCols ? vdim : kBlockCols;
+        chunk = 1;
+    }
     if (sequences < 0 || tokens < 0 || heads <= 0 || heads > 65535 || dim <= 0 || vdim <= 0 || groups <= 0 || chunk <= 0 ||
         parts <= 0 || slice <= 0 || slice > vdim || rot < 0 || rot % 2 || rot > dim ||
         (rot > 0 && (!cos_table || !sin_table)) || !(eps > 0.f) ||
@@ -430,9 +630,15 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
     const int padded = rows * parts;
     const size_t lds = sizeof(float) * static_cast<size_t>(chunk) *
                        (2 * static_cast<size_t>(rows) + slice + static_cast<size_t>(groups) * slice);
-    if (threads > 512 || lds > 64 * 1024 || static_cast<long>(slices) * parts > 65535 ||
-        static_cast<long>(chunk) * 2 * rows / 4 > static_cast<long>(kFetchPieces) * threads ||
-        static_cast<long>(chunk) * slice > static_cast<long>(kFetchValues) * threads)
+    if (!blocks && (threads > 512 || lds > 64 * 1024 || static_cast<long>(slices) * parts > 65535 ||
+                    static_cast<long>(chunk) * 2 * rows / 4 > static_cast<long>(kFetchPieces) * threads ||
+                    static_cast<long>(chunk) * slice > static_cast<long>(kFetchValues) * threads))
+        return CIE_BAD_ARGUMENT;
+    const size_t blocks_lds = sizeof(float) * (2 * static_cast<size_t>(kBlockTokens) * (padded + 4) + kBlockTokens * kBlockCols +
+                                               kBlockTokens * kScoreStride + 4 * kBlockTokens * kBlockCols + 36);
+    const int value_slices = (vdim + kBlockCols - 1) / kBlockCols;
+    if (blocks && (padded > 256 || blocks_lds > 64 * 1024 || value_slices > 65535 ||
+                   static_cast<long>(sequences) * heads > 0x7fffffffL))
         return CIE_BAD_ARGUMENT;
     if (sequences == 0 || tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -448,24 +654,46 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
                                                             sin_table, rot, positions, turned, heads, dim, padded, key_scale, act);
     else
         return CIE_BAD_ARGUMENT;
-    dim3 grid(sequences, heads, slices * parts);
     const long plane = static_cast<long>(tokens) * heads * vdim;
     int code = CIE_BAD_ARGUMENT;
-#define CIE_RETENTION(T, DS)                                                                                         \
-    code = launch_retention<T, DS>(s, grid, threads, lds, proj, ldp, v_off, turned, decay, state, seq_slot,          \
-                                   q_start_loc, raw, plane, heads, dim, vdim, slice, slices, groups, padded, chunk, act)
-    if (dtype == CIE_F32) {
-        if (rows_per_thread == 4) CIE_RETENTION(float, 4);
-        else if (rows_per_thread == 8) CIE_RETENTION(float, 8);
-        else if (rows_per_thread == 16) CIE_RETENTION(float, 16);
-        else if (rows_per_thread == 32) CIE_RETENTION(float, 32);
+    if (blocks) {
+        // (the workgroups of one head follow each other at a distance of `sequences * heads`: where that is a multiple
+        // of eight they share an XCD, and its L2 holds the head's queries and keys for all of them)
+        const dim3 block_grid(sequences * heads, value_slices);
+#define CIE_BLOCKS(T, TPW)                                                                                            \
+    retention_blocks_kernel<T, TPW><<<block_grid, 256, blocks_lds, s>>>(static_cast<const T*>(proj), ldp, v_off, turned,   \
+                                                                          decay, state, seq_slot, q_start_loc, raw, heads, \
+                                                                          dim, vdim, padded, act)
+        if (dtype == CIE_F32) {
+            if (padded <= 64) CIE_BLOCKS(float, 1);
+            else if (padded <= 128) CIE_BLOCKS(float, 2);
+            else CIE_BLOCKS(float, 4);
+        } else {
+            if (padded <= 64) CIE_BLOCKS(bf16_t, 1);
+            else if (padded <= 128) CIE_BLOCKS(bf16_t, 2);
+            else CIE_BLOCKS(bf16_t, 4);
+        }
+#undef CIE_BLOCKS
+        code = cie_after_launch();
+        parts = 1;
     } else {
-        if (rows_per_thread == 4) CIE_RETENTION(bf16_t, 4);
-        else if (rows_per_thread == 8) CIE_RETENTION(bf16_t, 8);
-        else if (rows_per_thread == 16) CIE_RETENTION(bf16_t, 16);
-        else if (rows_per_thread == 32) CIE_RETENTION(bf16_t, 32);
-    }
+        dim3 grid(sequences, heads, slices * parts);
+#define CIE_RETENTION(T, DS)                                                                                         \
+        code = launch_retention<T, DS>(s, grid, threads, lds, proj, ldp, v_off, turned, decay, state, seq_slot,          \
+                                       q_start_loc, raw, plane, heads, dim, vdim, slice, slices, groups, padded, chunk, act)
+        if (dtype == CIE_F32) {
+            if (rows_per_thread == 4) CIE_RETENTION(float, 4);
+            else if (rows_per_thread == 8) CIE_RETENTION(float, 8);
+            else if (rows_per_thread == 16) CIE_RETENTION(float, 16);
+            else if (rows_per_thread == 32) CIE_RETENTION(float, 32);
+        } else {
+            if (rows_per_thread == 4) CIE_RETENTION(bf16_t, 4);
+            else if (rows_per_thread == 8) CIE_RETENTION(bf16_t, 8);
+            else if (rows_per_thread == 16) CIE_RETENTION(bf16_t, 16);
+            else if (rows_per_thread == 32) CIE_RETENTION(bf16_t, 32);
+        }
 #undef CIE_RETENTION
+    }
     if (code != CIE_OK) return code;
     const int items = tokens * (heads / norm_span);
     const int width = norm_span * vdim;
@@ -483,13 +711,13 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
                 eps, norm_span, norm_weight, gate_act);
         return cie_after_launch();
     }
-    const int blocks = (items + 3) / 4;
+    const int norm_blocks = (items + 3) / 4;
     if (dtype == CIE_F32)
-        retention_norm_kernel<float><<<blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const float*>(proj), ldp, g_off,
+        retention_norm_kernel<float><<<norm_blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const float*>(proj), ldp, g_off,
                                                            static_cast<float*>(out), tokens, heads, vdim, eps, norm_span,
                                                            norm_weight, gate_act);
     else
-        retention_norm_kernel<bf16_t><<<blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const bf16_t*>(proj), ldp, g_off,
+        retention_norm_kernel<bf16_t><<<norm_blocks, 256, 0, s>>>(raw, plane, parts, static_cast<const bf16_t*>(proj), ldp, g_off,
                                                             static_cast<bf16_t*>(out), tokens, heads, vdim, eps, norm_span,
                                                             norm_weight, gate_act);
     return cie_after_launch();

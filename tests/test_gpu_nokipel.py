@@ -78,6 +78,11 @@ MECHANISMS = {
                             "mixer": {"heads": 3, "dim": 40, "vdim": 8, "decay": [0.5, 0.9, 0.999]}},
     "lightning_heads_of_64": {"type": "lightning", "mlp": None,
                               "mixer": {"heads": 2, "dim": 64, "vdim": 64, "decay": [0.75, 0.998046875]}},
+    # keys of more than 64 and of more than 128 numbers: more tiles of the memory's rows a wave in the walk by blocks
+    "lightning_heads_of_128": {"type": "lightning", "mlp": None,
+                               "mixer": {"heads": 2, "dim": 128, "vdim": 128, "decay": [0.9375, 0.99951171875]}},
+    "lightning_long_keys": {"type": "lightning", "mlp": None,
+                            "mixer": {"heads": 1, "dim": 160, "vdim": 24, "decay": [0.984375]}},
     # rows of all heads' read-outs wider than one wave norms: 1,080 and 2,176 numbers
     "lightning_wide_rows": {"type": "lightning", "mlp": None,
                             "mixer": {"heads": 9, "dim": 4, "vdim": 120, "decay": [0.5 + 0.055 * h for h in range(9)]}},
