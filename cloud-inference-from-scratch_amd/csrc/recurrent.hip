@@ -104,8 +104,7 @@ constexpr int kFetchValues = 12; // ... and values
             const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * slice - 1);                 \
             const int t = idx / slice;                                                                                \
             const int c = min(v0 + idx - t * slice, vdim - 1);                                                        \
-            ahead_v[i] = activated(                                                                                   \
-                to_float(proj[static_cast<size_t>(first + (from) + t) * ldp + v_off + head * vdim + c]), act);        \
+            ahead_v[i] = proj[static_cast<size_t>(first + (from) + t) * ldp + v_off + head * vdim + c];               \
         }                                                                                                             \
     }
 
@@ -141,7 +140,7 @@ retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* _
 #pragma unroll
     for (int r = 0; r < DS; ++r) S[r] = (owner && d0 + r < dim) ? mem[static_cast<size_t>(d0 + r) * vdim] : 0.f;
     piece_t ahead[kFetchPieces];
-    float ahead_v[kFetchValues];
+    T ahead_v[kFetchValues];  // (as stored: a conversion right behind the load would wait for it, and for all loads before it)
     if (count > 0) CIE_RETENTION_FETCH(0)
     for (int c0 = 0; c0 < count; c0 += chunk) {
         const int cn = min(chunk, count - c0);
@@ -153,7 +152,7 @@ retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* _
 #pragma unroll
         for (int i = 0; i < kFetchValues; ++i) {
             const int idx = threadIdx.x + i * blockDim.x;
-            if (idx < cn * slice) v_s[idx] = ahead_v[i];
+            if (idx < cn * slice) v_s[idx] = activated(to_float(ahead_v[i]), act);
         }
         __syncthreads();
         if (c0 + chunk < count) CIE_RETENTION_FETCH(c0 + chunk)
@@ -217,6 +216,15 @@ retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* _
 }
 #undef CIE_RETENTION_FETCH
 
+// A barrier for what the waves of a workgroup hand each other through LDS.  It waits for the wave's LDS traffic only:
+// loads from memory that are under way stay under way (`__syncthreads` waits for them too, which would put a block's
+// way from memory in front of every barrier of a loop that fetches a block ahead).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // (b') The same walk for sequences that bring many tokens (a prompt's portion), in blocks of 32 tokens on the matrix
 // cores, float32 throughout (`v_mfma_f32_16x16x4_f32`: operands and sums are plain float32).  With S the memory in
 // front of a block, i and j tokens of the block and f the head's decay:
@@ -269,75 +277,106 @@ retention_blocks_kernel(const T* __restrict__ proj, long ldp, int v_off, const f
             f *= fade;
         }
     }
-    // rows of S: lane (g, l16), number r of tile t holds row 16 t + 4 r + g of column v0 + l16
+    // rows of S: lane (g, l16), number r of tile t holds row 16 t + 4 g + r of column v0 + l16 (the result layout)
     float* mem = state + ((static_cast<size_t>(slot) * heads + head) * dim) * vdim + v0 + l16;
     acc4_t S[TPW];
 #pragma unroll
     for (int u = 0; u < TPW; ++u)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int row = 16 * (wave * TPW + u) + 4 * r + g;
+            const int row = 16 * (wave * TPW + u) + 4 * g + r;
             S[u][r] = (col_ok && row < dim) ? mem[static_cast<size_t>(row) * vdim] : 0.f;
         }
+    // which pieces of a block this thread fetches and where they go in LDS does not change from block to block
+    // (divisions by sizes that only the launch knows: made once, not per block)
     const int pieces = padded / 2;                       // 16-byte pieces of one token's query and key
+    int piece_token[4 * TPW], piece_from[4 * TPW], piece_to[4 * TPW];
+#pragma unroll
+    for (int i = 0; i < 4 * TPW; ++i) {
+        const int idx = min(static_cast<int>(threadIdx.x) + i * 256, kBlockTokens * pieces - 1);
+        const int t = idx / pieces;
+        const int within = idx - t * pieces;
+        const int side = within / (padded / 4);          // 0: the query, 1: the key
+        piece_token[i] = t;
+        piece_from[i] = within * 4;
+        piece_to[i] = (side ? kBlockTokens * stride : 0) + t * stride + (within - side * (padded / 4)) * 4;
+    }
+    const T* values = proj + v_off + head * vdim;
     piece_t ahead[4 * TPW];
-    float ahead_v[2];
+    T ahead_v[2];  // (as stored: a conversion right behind the load would wait for it, and for all loads before it)
 #define CIE_BLOCKS_FETCH(from)                                                                                        \
     {                                                                                                                 \
-        const int fetch_n = min(kBlockTokens, count - (from));                                                        \
-        _Pragma("unroll") for (int i = 0; i < 4 * TPW; ++i) {                                                         \
-            const int idx = min(static_cast<int>(threadIdx.x) + i * 256, fetch_n * pieces - 1);                       \
-            const int t = idx / pieces;                                                                               \
+        const int last = min(kBlockTokens, count - (from)) - 1;                                                       \
+        const float* base = turned + (static_cast<size_t>(first + (from)) * heads + head) * 2 * padded;               \
+        _Pragma("unroll") for (int i = 0; i < 4 * TPW; ++i)                                                           \
             ahead[i] = *reinterpret_cast<const piece_t*>(                                                             \
-                turned + (static_cast<size_t>(first + (from) + t) * heads + head) * 2 * padded + (idx - t * pieces) * 4); \
-        }                                                                                                             \
+                base + static_cast<size_t>(min(piece_token[i], last)) * heads * 2 * padded + piece_from[i]);          \
         _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                               \
             const int idx = static_cast<int>(threadIdx.x) + i * 256;                                                  \
-            const int t = min(idx / kBlockCols, fetch_n - 1);                                                         \
+            const int t = min(idx / kBlockCols, last);                                                                \
             const int c = min(v0 + idx % kBlockCols, vdim - 1);                                                       \
-            ahead_v[i] = activated(                                                                                   \
-                to_float(proj[static_cast<size_t>(first + (from) + t) * ldp + v_off + head * vdim + c]), act);        \
+            ahead_v[i] = values[static_cast<size_t>(first + (from) + t) * ldp + c];                                   \
         }                                                                                                             \
     }
+    // the powers of the decay that this lane applies: they depend on its place, and on the block's length
+    lds_barrier();                                       // (the table)
+    const int ti = wave >> 1, tj = wave & 1;             // this wave's tile of the scores
+    float p_fade[4], o_fade[2][4], k_fade[kBlockTokens / 4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int apart = 16 * (ti - tj) + 4 * g + r - l16;  // i - j
+        p_fade[r] = apart >= 0 ? pw[min(apart, kBlockTokens)] : 0.f;
+        o_fade[0][r] = pw[4 * g + r + 1];
+        o_fade[1][r] = pw[16 + 4 * g + r + 1];
+    }
+    int faded_for = -1;
+    float keep = 0.f;
     if (count > 0) CIE_BLOCKS_FETCH(0)
     for (int c0 = 0; c0 < count; c0 += kBlockTokens) {
         const int cn = min(kBlockTokens, count - c0);
+        if (cn != faded_for) {                           // (the first block, and a last one that is shorter)
+            faded_for = cn;
+            keep = pw[cn];
+#pragma unroll
+            for (int kk = 0; kk < kBlockTokens / 4; ++kk) k_fade[kk] = pw[max(cn - 1 - (4 * kk + g), 0)];
+        }
         // the block into LDS; rows past the block's last token are zero
 #pragma unroll
-        for (int i = 0; i < 4 * TPW; ++i) {
-            const int idx = threadIdx.x + i * 256;
-            if (idx < kBlockTokens * pieces) {
-                const int t = idx / pieces;
-                const int within = idx - t * pieces;
-                const int side = within / (padded / 4);  // 0: the query, 1: the key
-                const piece_t value = t < cn ? ahead[i] : piece_t{0.f, 0.f, 0.f, 0.f};
-                *reinterpret_cast<piece_t*>((side ? k_s : q_s) + t * stride + (within - side * (padded / 4)) * 4) = value;
-            }
-        }
+        for (int i = 0; i < 4 * TPW; ++i)
+            if (static_cast<int>(threadIdx.x) + i * 256 < kBlockTokens * pieces)
+                *reinterpret_cast<piece_t*>(lds + piece_to[i]) =
+                    piece_token[i] < cn ? ahead[i] : piece_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int idx = threadIdx.x + i * 256;
-            const int t = idx / kBlockCols;
-            v_s[idx] = (t < cn && v0 + idx % kBlockCols < vdim) ? ahead_v[i] : 0.f;
+            v_s[idx] = (idx / kBlockCols < cn && v0 + idx % kBlockCols < vdim) ? activated(to_float(ahead_v[i]), act) : 0.f;
         }
-        __syncthreads();
+        lds_barrier();
         if (c0 + kBlockTokens < count) CIE_BLOCKS_FETCH(c0 + kBlockTokens)
         // this wave's tile of the scores
         {
-            const int ti = wave >> 1, tj = wave & 1;
             acc4_t p = {0.f, 0.f, 0.f, 0.f};
             if (tj <= ti) {
-                const float* qa = q_s + (16 * ti + l16) * stride + g;
-                const float* kb = k_s + (16 * tj + l16) * stride + g;
-                for (int kk = 0; kk < padded / 4; ++kk)
-                    p = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[4 * kk], kb[4 * kk], p, 0, 0, 0);
-            }
-            const int j = 16 * tj + l16;
+                // (a lane reads four neighbouring numbers at once and spends them on four products: which four
+                // numbers of the sum a product takes does not matter as long as both operands agree)
+                const float* qa = q_s + (16 * ti + l16) * stride + 4 * g;
+                const float* kb = k_s + (16 * tj + l16) * stride + 4 * g;
+                acc4_t p1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int i = 16 * ti + 4 * g + r;
-                p_s[i * kScoreStride + j] = j <= i ? p[r] * pw[i - j] : 0.f;
+                for (int m = 0; m < 4 * TPW; ++m) {
+                    if (m >= tiles) break;
+                    const float4 a = *reinterpret_cast<const float4*>(qa + 16 * m);
+                    const float4 b = *reinterpret_cast<const float4*>(kb + 16 * m);
+                    p = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, p, 0, 0, 0);
+                    p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, p1, 0, 0, 0);
+                    p = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, p, 0, 0, 0);
+                    p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, p1, 0, 0, 0);
+                }
+                p += p1;
             }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                p_s[(16 * ti + 4 * g + r) * kScoreStride + 16 * tj + l16] = p[r] * p_fade[r];
         }
         // this wave's share of S^T q, faded by the tokens' places in the block
         acc4_t o[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
@@ -345,19 +384,23 @@ retention_blocks_kernel(const T* __restrict__ proj, long ldp, int v_off, const f
         for (int u = 0; u < TPW; ++u) {
             const int t = wave * TPW + u;
             if (t < tiles) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int d = 16 * t + 4 * r + g;
-                    o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(q_s[l16 * stride + d], S[u][r], o[0], 0, 0, 0);
-                    o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(q_s[(16 + l16) * stride + d], S[u][r], o[1], 0, 0, 0);
-                }
+                const float4 a0 = *reinterpret_cast<const float4*>(q_s + l16 * stride + 16 * t + 4 * g);
+                const float4 a1 = *reinterpret_cast<const float4*>(q_s + (16 + l16) * stride + 16 * t + 4 * g);
+                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.x, S[u][0], o[0], 0, 0, 0);
+                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.x, S[u][0], o[1], 0, 0, 0);
+                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.y, S[u][1], o[0], 0, 0, 0);
+                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.y, S[u][1], o[1], 0, 0, 0);
+                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.z, S[u][2], o[0], 0, 0, 0);
+                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.z, S[u][2], o[1], 0, 0, 0);
+                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.w, S[u][3], o[0], 0, 0, 0);
+                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.w, S[u][3], o[1], 0, 0, 0);
             }
         }
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o[rt][r] *= pw[16 * rt + 4 * g + r + 1];
-        __syncthreads();
+            for (int r = 0; r < 4; ++r) o[rt][r] *= o_fade[rt][r];
+        lds_barrier();
         // ... of the block's own sum: tokens 8 w .. 8 w + 7
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
@@ -373,8 +416,6 @@ retention_blocks_kernel(const T* __restrict__ proj, long ldp, int v_off, const f
                 red[(wave * kBlockTokens + 16 * rt + 4 * g + r) * kBlockCols + l16] = o[rt][r];
         // ... and of the new S
         {
-            const float keep = pw[cn];
-            const int mine = 4 * (l16 % 4) + l16 / 4;    // the row of a tile that stands at place l16 of the layout
 #pragma unroll
             for (int u = 0; u < TPW; ++u) {
                 const int t = wave * TPW + u;
@@ -384,13 +425,13 @@ retention_blocks_kernel(const T* __restrict__ proj, long ldp, int v_off, const f
 #pragma unroll
                     for (int kk = 0; kk < kBlockTokens / 4; ++kk) {
                         const int j = 4 * kk + g;
-                        const float ka = k_s[j * stride + 16 * t + mine] * pw[max(cn - 1 - j, 0)];
+                        const float ka = k_s[j * stride + 16 * t + l16] * k_fade[kk];
                         S[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka, v_s[j * kBlockCols + l16], S[u], 0, 0, 0);
                     }
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
         for (int idx = threadIdx.x; idx < cn * kBlockCols; idx += blockDim.x) {
             const int c = idx % kBlockCols;
             if (v0 + c >= vdim) continue;
@@ -404,7 +445,7 @@ retention_blocks_kernel(const T* __restrict__ proj, long ldp, int v_off, const f
     for (int u = 0; u < TPW; ++u)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int row = 16 * (wave * TPW + u) + 4 * r + g;
+            const int row = 16 * (wave * TPW + u) + 4 * g + r;
             if (col_ok && row < dim) mem[static_cast<size_t>(row) * vdim] = S[u][r];
         }
 }
