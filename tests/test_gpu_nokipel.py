@@ -66,8 +66,8 @@ MECHANISMS = {
     "attention_plain": {"type": "attention", "mlp": None, "mixer": {"heads": 2, "dim": 12, "vdim": 20, "scale": 0.5}},
     # head sizes of the matrix-core kernels
     "attention_heads_of_64": {"type": "attention", "mlp": None,
-                              "mixer": {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.15, "mask": {"size": 33},
-                                        "rot": {"base": 500000.0, "dims": 32}}},
+                              "mixer": {"heads": 6, "kv_heads": 3, "dim": 64, "vdim": 64, "scale": 0.15, "mask": {"size": 33},
+                                        "rot": {"base": 300000.0, "dims": 32}}},
     "attention_heads_of_128_and_64": {"type": "attention", "mlp": None,
                                       "mixer": {"heads": 2, "kv_heads": 1, "dim": 128, "vdim": 64, "scale": 0.1,
                                                 "mask": {"size": 40}, "rot": {"base": 10000.0, "dims": 128}}},
@@ -218,6 +218,64 @@ def test_random_traces_reuse_pages_and_slots(models, name, dtype):
     assert set(rows) <= set(requests) and rows
     worst, _ = nu.spread(rows, plain)
     assert worst <= LIMIT[dtype], worst
+
+
+def random_configuration(rng: random.Random) -> dict:
+    """A model whose every size, count, constant and layer order is drawn: widths and heads that are and are not
+    multiples of 8 or 64, chunks shorter than a page and longer than any request, loops anywhere."""
+    groups = rng.choice([2, 3, 4, 6])
+    width = groups * rng.choice([8, 12, 16, 20, 32])
+    layers = []
+    for _ in range(rng.randint(2, 6)):
+        if rng.random() < 0.5:
+            heads = rng.choice([1, 2, 3, 5])
+            mixer = {"heads": heads, "dim": rng.choice([4, 8, 24, 64, 72, 136]), "vdim": rng.choice([8, 16, 40, 64, 128]),
+                     "decay": [rng.choice([0.25, 0.75, 0.9375, 0.99609375, 0.9990234375]) for _ in range(heads)]}
+            kind = "lightning"
+        else:
+            kv_heads = rng.choice([1, 2, 3])
+            dim = rng.choice([8, 16, 24, 64, 128])
+            mixer = {"heads": kv_heads * rng.choice([1, 2, 4]), "kv_heads": kv_heads, "dim": dim,
+                     "vdim": rng.choice([8, 24, 64, 128]), "scale": rng.choice([0.5, 1.0, 2.0]) * dim ** -0.5,
+                     "mask": {"size": rng.choice([1, 3, 16, 17, 31, 64, 500])},
+                     "rot": {"base": rng.choice([10.0, 1000.0, 2.0e5]), "dims": rng.choice([d for d in (2, 4, 8, 16, 64, 128) if d <= dim])}}
+            kind = "attention"
+        draw = rng.random()
+        if draw < 0.15:
+            mlp = None
+        elif draw < 0.5:
+            mlp = {"kind": "dense", "ff": rng.choice([24, 52, 100]), "limit": rng.choice([0.5, 1.0, 4.0])}
+        else:
+            count, per = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 3, 5])
+            outputs = count * per
+            identity = rng.randint(0, min(outputs - 1, 3))
+            keep = rng.randint(1, count)
+            mlp = {"kind": "moe", "expert": {"ff": rng.choice([8, 20, 48])}, "shared": {"ff": rng.choice([8, 28])},
+                   "router": {"experts": outputs - identity, "identity": identity, "top": rng.randint(1, min(keep * per, 6)),
+                              "scale": rng.choice([0.5, 1.0, 2.5]), "groups": {"count": count, "keep": keep}}}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    start = rng.randint(0, len(layers) - 1)
+    return {"architecture": "Nokipel", "vocab": rng.choice([70, 130, 300]), "width": width,
+            "norm": {"eps": rng.choice([1e-6, 1e-5, 1e-3]), "groups": groups}, "embedding": {"scale": rng.choice([0.5, 2.0, 8.0])},
+            "loop": {"start": start, "stop": rng.randint(start, len(layers)), "times": rng.randint(1, 3)}, "layers": layers}
+
+
+@pytest.mark.filterwarnings("ignore:bfloat16 attention")
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations_and_traces(seed):
+    """Ten models that nobody chose, each under a random trace of six requests on three slots, in both precisions."""
+    rng = random.Random(1000 + seed)
+    raw = random_configuration(rng)
+    weights = nu.make_weights(raw, seed=seed, exact_router=True)
+    requests, steps = replay_util.random_trace(rng, [rng.choice([1, 2, 9, 33, 48, 70]) for _ in range(6)], raw["vocab"], 16, live_most=3)
+    plain = plain_all(raw, weights, requests)
+    for dtype in ("float32", "bfloat16"):
+        runner = nu.make_runner(raw, weights, dtype, max(replay_util.max_live_tokens(steps, page=16), 16), 16, 3)
+        rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
+        assert rows
+        worst, _ = nu.spread(rows, plain)
+        assert worst <= LIMIT[dtype], (dtype, worst, raw)
+        assert runner.cache.stats().slots_used == 0 and runner.cache.stats().pages_used == 0
 
 
 NEEDLE, ASK, FILLERS = 1, 2, 40  # token ids: the one to be found, the one that looks for it, the first of the rest
