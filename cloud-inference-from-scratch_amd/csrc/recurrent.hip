@@ -216,238 +216,250 @@ retention_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* _
 }
 #undef CIE_RETENTION_FETCH
 
-// A barrier for what the waves of a workgroup hand each other through LDS.  It waits for the wave's LDS traffic only:
-// loads from memory that are under way stay under way (`__syncthreads` waits for them too, which would put a block's
-// way from memory in front of every barrier of a loop that fetches a block ahead).
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-// (b') The same walk for sequences that bring many tokens (a prompt's portion), in blocks of 32 tokens on the matrix
-// cores, float32 throughout (`v_mfma_f32_16x16x4_f32`: operands and sums are plain float32).  With S the memory in
-// front of a block, i and j tokens of the block and f the head's decay:
+// (b') The same walk for sequences that bring many tokens (a prompt's portion): blocks of 32 tokens on the matrix
+// cores, float32 throughout (`v_mfma_f32_16x16x4_f32`: operands and sums are plain float32), and only what has to
+// wait for the block before it waits.  With S the memory in front of a block of n tokens, i and j tokens of the
+// block and f the head's decay:
 //     o_i   = f^(i+1) * (S^T q_i)  +  sum_{j <= i} f^(i-j) (q_i . k_j) v_j
-//     S_new = f^n * S  +  sum_j f^(n-1-j) k_j v_j^T          (n the block's tokens: 32, or fewer at the end)
-// One workgroup of four waves takes (sequence, head, 16 value columns) and walks the blocks in order.  The block's
-// queries, keys and values wait in LDS (fetched into registers a block ahead).  Wave w keeps rows of S in the matrix
-// cores' result layout, where they serve as the second operand of S^T q as they are; it makes one 16 x 16 tile of
-// q . k (the tile above the diagonal is zero), and its share of S^T q, of the block's own sum (tokens 8w .. 8w + 7)
-// and of the new S; the waves' shares of o meet in LDS in the waves' order.  Powers of f come from a table made by
-// repeated multiplication, as the walk token by token makes them.
+//     S_new = f^n * S  +  sum_j f^(n-1-j) k_j v_j^T
+// Three kernels.  `retention_block_sums_kernel`, every block at once: the second term of o (into the first plane of
+// `raw`) and the second term of S_new (into the block's place of `sums`).  `retention_scan_kernel`, one thread per
+// number of the memory, over a sequence's blocks in order: the block's place gets the S in front of it, and S moves on.
+// `retention_block_reads_kernel`, every block at once: the first term of o (into the second plane).  The norm kernel
+// adds the planes.  Block b of sequence s has place first_token(s) / 32 + s + b: no two blocks share one, and there
+// are at most tokens / 32 + sequences + 1 places.  Queries and keys are the turn kernel's float32 rows, padded to whole
+// tiles of 16; a workgroup takes up to 128 value columns (a panel), rounded up to tiles of 16 (`vdim16` columns a row
+// of `sums`).  Operand layouts of the 16 x 16 x 4 product: lane (l16 = lane % 16, g = lane / 16) gives A[l16][g] and
+// B[g][l16] and gets rows 4 g .. 4 g + 3 of column l16; which four numbers of a sum a product takes does not matter
+// as long as both operands agree, so a lane reads four neighbouring numbers at once and spends them on four products.
 typedef float acc4_t __attribute__((ext_vector_type(4)));
 constexpr int kBlockTokens = 32;
-constexpr int kBlockCols = 16;
+constexpr int kPanelCols = 128;
 constexpr int kScoreStride = kBlockTokens + 4;
 
-// TPW: tiles of 16 rows of S that a wave keeps (the head's `padded` numbers are at most 64 * TPW)
-template <typename T, int TPW>
-__global__ void __launch_bounds__(256)
-retention_blocks_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* __restrict__ turned,
-                        const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ seq_slot,
-                        const int* __restrict__ q_start_loc, float* __restrict__ raw, int heads, int dim, int vdim,
-                        int padded, int act) {
-    extern __shared__ float4 lds4[];
-    float* lds = reinterpret_cast<float*>(lds4);
-    const int stride = padded + 4;                       // (a row's start moves on by four banks)
-    float* q_s = lds;                                    // [32][stride]
-    float* k_s = q_s + kBlockTokens * stride;            // [32][stride]
-    float* v_s = k_s + kBlockTokens * stride;            // [32][16]
-    float* p_s = v_s + kBlockTokens * kBlockCols;        // [32][36]: f^(i-j) (q_i . k_j), zero above the diagonal
-    float* red = p_s + kBlockTokens * kScoreStride;      // [4][32][16]: the waves' shares of o
-    float* pw = red + 4 * kBlockTokens * kBlockCols;     // [33]: powers of the decay
-    const int seq = blockIdx.x / heads;
-    const int head = blockIdx.x - seq * heads;
-    const int v0 = blockIdx.y * kBlockCols;
-    const int first = q_start_loc[seq];
-    const int count = q_start_loc[seq + 1] - first;
-    const int slot = seq_slot[seq];
-    const int lane = threadIdx.x % kWave;
-    const int wave = threadIdx.x / kWave;
-    const int l16 = lane % 16;
-    const int g = lane / 16;
-    const int tiles = padded / 16;
-    const bool col_ok = v0 + l16 < vdim;
+// rows of a panel of values in LDS start 16 banks apart: the four tokens that a product reads then touch every bank
+__host__ __device__ inline int panel_stride(int cols) { return cols % 32 == 0 ? cols + 16 : cols; }
+
+// powers of the decay by repeated multiplication, as the walk token by token makes them
+__device__ __forceinline__ void decay_table(float* pw, float fade) {
     if (threadIdx.x == 0) {
         float f = 1.0f;
-        const float fade = decay[head];
         for (int n = 0; n <= kBlockTokens; ++n) {
             pw[n] = f;
             f *= fade;
         }
     }
-    // rows of S: lane (g, l16), number r of tile t holds row 16 t + 4 g + r of column v0 + l16 (the result layout)
-    float* mem = state + ((static_cast<size_t>(slot) * heads + head) * dim) * vdim + v0 + l16;
-    acc4_t S[TPW];
-#pragma unroll
-    for (int u = 0; u < TPW; ++u)
+}
+
+// a block's queries (side 0) or keys (side 1) into LDS rows of `stride` floats; rows past the block's last token are zero
+__device__ __forceinline__ void stage_rows(float* dst, int stride, const float* __restrict__ turned, int first_token,
+                                           int cn, int heads, int head, int padded, int side) {
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    for (int t = wave; t < kBlockTokens; t += 4) {
+        const float* src = turned + ((static_cast<size_t>(first_token + min(t, cn - 1)) * heads + head) * 2 + side) * padded;
+        for (int piece = lane; piece < padded / 4; piece += kWave) {
+            const piece_t value = *reinterpret_cast<const piece_t*>(src + 4 * piece);
+            *reinterpret_cast<piece_t*>(dst + t * stride + 4 * piece) = t < cn ? value : piece_t{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+retention_block_sums_kernel(const T* __restrict__ proj, long ldp, int v_off, const float* __restrict__ turned,
+                            const float* __restrict__ decay, const int* __restrict__ q_start_loc,
+                            float* __restrict__ raw, float* __restrict__ sums, int heads, int vdim, int padded,
+                            int vdim16, int act) {
+    const int seq = blockIdx.x / heads;
+    const int head = blockIdx.x - seq * heads;
+    const int first = q_start_loc[seq];
+    const int count = q_start_loc[seq + 1] - first;
+    const int c0 = blockIdx.y * kBlockTokens;
+    if (c0 >= count) return;                             // (the whole workgroup: the grid is sized for the longest sequence)
+    const int cn = min(kBlockTokens, count - c0);
+    const int panel0 = blockIdx.z * kPanelCols;
+    const int cols = min(kPanelCols, vdim16 - panel0);
+    const int col_tiles = cols / 16;
+    const int stride = padded + 4;
+    const int vstride = panel_stride(cols);
+    extern __shared__ float4 lds4[];
+    float* q_s = reinterpret_cast<float*>(lds4);          // [32][stride]
+    float* k_s = q_s + kBlockTokens * stride;            // [32][stride]
+    float* v_s = k_s + kBlockTokens * stride;            // [32][vstride]
+    float* p_s = v_s + kBlockTokens * vstride;           // [32][36]: f^(i-j) (q_i . k_j), zero above the diagonal
+    float* pw = p_s + kBlockTokens * kScoreStride;       // [33]
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int l16 = lane % 16;
+    const int g = lane / 16;
+    const int tiles = padded / 16;
+    decay_table(pw, decay[head]);
+    stage_rows(q_s, stride, turned, first + c0, cn, heads, head, padded, 0);
+    stage_rows(k_s, stride, turned, first + c0, cn, heads, head, padded, 1);
+    for (int t = wave; t < kBlockTokens; t += 4) {
+        const T* src = proj + static_cast<size_t>(first + c0 + min(t, cn - 1)) * ldp + v_off + head * vdim;
+        for (int c = lane; c < cols; c += kWave) {
+            const float value = activated(to_float(src[min(panel0 + c, vdim - 1)]), act);
+            v_s[t * vstride + c] = (t < cn && panel0 + c < vdim) ? value : 0.f;
+        }
+    }
+    __syncthreads();
+    {   // this wave's tile of the scores (the tile above the diagonal is zero)
+        const int ti = wave >> 1, tj = wave & 1;
+        acc4_t p = {0.f, 0.f, 0.f, 0.f};
+        if (tj <= ti) {
+            const float* qa = q_s + (16 * ti + l16) * stride + 4 * g;
+            const float* kb = k_s + (16 * tj + l16) * stride + 4 * g;
+            acc4_t p1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+            for (int m = 0; m < tiles; ++m) {
+                const float4 a = *reinterpret_cast<const float4*>(qa + 16 * m);
+                const float4 b = *reinterpret_cast<const float4*>(kb + 16 * m);
+                p = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, p, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, p1, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, p, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, p1, 0, 0, 0);
+            }
+            p += p1;
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int row = 16 * (wave * TPW + u) + 4 * g + r;
-            S[u][r] = (col_ok && row < dim) ? mem[static_cast<size_t>(row) * vdim] : 0.f;
+            const int apart = 16 * (ti - tj) + 4 * g + r - l16;  // i - j
+            p_s[(16 * ti + 4 * g + r) * kScoreStride + 16 * tj + l16] = apart >= 0 ? p[r] * pw[min(apart, kBlockTokens)] : 0.f;
         }
-    // which pieces of a block this thread fetches and where they go in LDS does not change from block to block
-    // (divisions by sizes that only the launch knows: made once, not per block)
-    const int pieces = padded / 2;                       // 16-byte pieces of one token's query and key
-    int piece_token[4 * TPW], piece_from[4 * TPW], piece_to[4 * TPW];
-#pragma unroll
-    for (int i = 0; i < 4 * TPW; ++i) {
-        const int idx = min(static_cast<int>(threadIdx.x) + i * 256, kBlockTokens * pieces - 1);
-        const int t = idx / pieces;
-        const int within = idx - t * pieces;
-        const int side = within / (padded / 4);          // 0: the query, 1: the key
-        piece_token[i] = t;
-        piece_from[i] = within * 4;
-        piece_to[i] = (side ? kBlockTokens * stride : 0) + t * stride + (within - side * (padded / 4)) * 4;
     }
-    const T* values = proj + v_off + head * vdim;
-    piece_t ahead[4 * TPW];
-    T ahead_v[2];  // (as stored: a conversion right behind the load would wait for it, and for all loads before it)
-#define CIE_BLOCKS_FETCH(from)                                                                                        \
-    {                                                                                                                 \
-        const int last = min(kBlockTokens, count - (from)) - 1;                                                       \
-        const float* base = turned + (static_cast<size_t>(first + (from)) * heads + head) * 2 * padded;               \
-        _Pragma("unroll") for (int i = 0; i < 4 * TPW; ++i)                                                           \
-            ahead[i] = *reinterpret_cast<const piece_t*>(                                                             \
-                base + static_cast<size_t>(min(piece_token[i], last)) * heads * 2 * padded + piece_from[i]);          \
-        _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                               \
-            const int idx = static_cast<int>(threadIdx.x) + i * 256;                                                  \
-            const int t = min(idx / kBlockCols, last);                                                                \
-            const int c = min(v0 + idx % kBlockCols, vdim - 1);                                                       \
-            ahead_v[i] = values[static_cast<size_t>(first + (from) + t) * ldp + c];                                   \
-        }                                                                                                             \
-    }
-    // the powers of the decay that this lane applies: they depend on its place, and on the block's length
-    lds_barrier();                                       // (the table)
-    const int ti = wave >> 1, tj = wave & 1;             // this wave's tile of the scores
-    float p_fade[4], o_fade[2][4], k_fade[kBlockTokens / 4];
+    __syncthreads();
+    float k_fade[kBlockTokens / 4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int apart = 16 * (ti - tj) + 4 * g + r - l16;  // i - j
-        p_fade[r] = apart >= 0 ? pw[min(apart, kBlockTokens)] : 0.f;
-        o_fade[0][r] = pw[4 * g + r + 1];
-        o_fade[1][r] = pw[16 + 4 * g + r + 1];
-    }
-    int faded_for = -1;
-    float keep = 0.f;
-    if (count > 0) CIE_BLOCKS_FETCH(0)
-    for (int c0 = 0; c0 < count; c0 += kBlockTokens) {
-        const int cn = min(kBlockTokens, count - c0);
-        if (cn != faded_for) {                           // (the first block, and a last one that is shorter)
-            faded_for = cn;
-            keep = pw[cn];
+    for (int kk = 0; kk < kBlockTokens / 4; ++kk) k_fade[kk] = pw[max(cn - 1 - (4 * kk + g), 0)];
+    const int place = first / kBlockTokens + seq + blockIdx.y;
+    float* sum_rows = sums + (static_cast<size_t>(place) * heads + head) * padded * vdim16 + panel0;
+    for (int ct = wave; ct < col_tiles; ct += 4) {       // this wave's tiles of value columns
+        float vb[kBlockTokens / 4];
 #pragma unroll
-            for (int kk = 0; kk < kBlockTokens / 4; ++kk) k_fade[kk] = pw[max(cn - 1 - (4 * kk + g), 0)];
+        for (int kk = 0; kk < kBlockTokens / 4; ++kk) vb[kk] = v_s[(4 * kk + g) * vstride + 16 * ct + l16];
+        // the block's own sum
+        acc4_t o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < kBlockTokens / 4; ++kk) {
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[l16 * kScoreStride + 4 * kk + g], vb[kk], o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[(16 + l16) * kScoreStride + 4 * kk + g], vb[kk], o1, 0, 0, 0);
         }
-        // the block into LDS; rows past the block's last token are zero
+        const int col = panel0 + 16 * ct + l16;
+        if (col < vdim) {
 #pragma unroll
-        for (int i = 0; i < 4 * TPW; ++i)
-            if (static_cast<int>(threadIdx.x) + i * 256 < kBlockTokens * pieces)
-                *reinterpret_cast<piece_t*>(lds + piece_to[i]) =
-                    piece_token[i] < cn ? ahead[i] : piece_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int idx = threadIdx.x + i * 256;
-            v_s[idx] = (idx / kBlockCols < cn && v0 + idx % kBlockCols < vdim) ? activated(to_float(ahead_v[i]), act) : 0.f;
-        }
-        lds_barrier();
-        if (c0 + kBlockTokens < count) CIE_BLOCKS_FETCH(c0 + kBlockTokens)
-        // this wave's tile of the scores
-        {
-            acc4_t p = {0.f, 0.f, 0.f, 0.f};
-            if (tj <= ti) {
-                // (a lane reads four neighbouring numbers at once and spends them on four products: which four
-                // numbers of the sum a product takes does not matter as long as both operands agree)
-                const float* qa = q_s + (16 * ti + l16) * stride + 4 * g;
-                const float* kb = k_s + (16 * tj + l16) * stride + 4 * g;
-                acc4_t p1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int m = 0; m < 4 * TPW; ++m) {
-                    if (m >= tiles) break;
-                    const float4 a = *reinterpret_cast<const float4*>(qa + 16 * m);
-                    const float4 b = *reinterpret_cast<const float4*>(kb + 16 * m);
-                    p = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b.x, p, 0, 0, 0);
-                    p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b.y, p1, 0, 0, 0);
-                    p = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b.z, p, 0, 0, 0);
-                    p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b.w, p1, 0, 0, 0);
-                }
-                p += p1;
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                p_s[(16 * ti + 4 * g + r) * kScoreStride + 16 * tj + l16] = p[r] * p_fade[r];
-        }
-        // this wave's share of S^T q, faded by the tokens' places in the block
-        acc4_t o[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-#pragma unroll
-        for (int u = 0; u < TPW; ++u) {
-            const int t = wave * TPW + u;
-            if (t < tiles) {
-                const float4 a0 = *reinterpret_cast<const float4*>(q_s + l16 * stride + 16 * t + 4 * g);
-                const float4 a1 = *reinterpret_cast<const float4*>(q_s + (16 + l16) * stride + 16 * t + 4 * g);
-                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.x, S[u][0], o[0], 0, 0, 0);
-                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.x, S[u][0], o[1], 0, 0, 0);
-                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.y, S[u][1], o[0], 0, 0, 0);
-                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.y, S[u][1], o[1], 0, 0, 0);
-                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.z, S[u][2], o[0], 0, 0, 0);
-                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.z, S[u][2], o[1], 0, 0, 0);
-                o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.w, S[u][3], o[0], 0, 0, 0);
-                o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.w, S[u][3], o[1], 0, 0, 0);
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * g + r;
+                float* dst = raw + static_cast<size_t>(first + c0) * heads * vdim + head * vdim + col;
+                if (i < cn) dst[static_cast<size_t>(i) * heads * vdim] = o0[r];
+                if (16 + i < cn) dst[static_cast<size_t>(16 + i) * heads * vdim] = o1[r];
             }
         }
+        // what the block adds to the memory
+        for (int rt = 0; rt < tiles; ++rt) {
+            acc4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt)
+            for (int kk = 0; kk < kBlockTokens / 4; ++kk)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(k_s[(4 * kk + g) * stride + 16 * rt + l16] * k_fade[kk], vb[kk],
+                                                          acc, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) o[rt][r] *= o_fade[rt][r];
-        lds_barrier();
-        // ... of the block's own sum: tokens 8 w .. 8 w + 7
-#pragma unroll
-        for (int kk = 0; kk < 2; ++kk) {
-            const int j = 8 * wave + 4 * kk + g;
-            const float vb = v_s[j * kBlockCols + l16];
-            o[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[l16 * kScoreStride + j], vb, o[0], 0, 0, 0);
-            o[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[(16 + l16) * kScoreStride + j], vb, o[1], 0, 0, 0);
-        }
-#pragma unroll
-        for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                red[(wave * kBlockTokens + 16 * rt + 4 * g + r) * kBlockCols + l16] = o[rt][r];
-        // ... and of the new S
-        {
-#pragma unroll
-            for (int u = 0; u < TPW; ++u) {
-                const int t = wave * TPW + u;
-                if (t < tiles) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) S[u][r] *= keep;
-#pragma unroll
-                    for (int kk = 0; kk < kBlockTokens / 4; ++kk) {
-                        const int j = 4 * kk + g;
-                        const float ka = k_s[j * stride + 16 * t + l16] * k_fade[kk];
-                        S[u] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka, v_s[j * kBlockCols + l16], S[u], 0, 0, 0);
-                    }
-                }
-            }
-        }
-        lds_barrier();
-        for (int idx = threadIdx.x; idx < cn * kBlockCols; idx += blockDim.x) {
-            const int c = idx % kBlockCols;
-            if (v0 + c >= vdim) continue;
-            float sum = red[idx];
-            for (int w = 1; w < 4; ++w) sum += red[w * kBlockTokens * kBlockCols + idx];
-            raw[static_cast<size_t>(first + c0 + idx / kBlockCols) * heads * vdim + head * vdim + v0 + c] = sum;
+            for (int r = 0; r < 4; ++r) sum_rows[static_cast<size_t>(16 * rt + 4 * g + r) * vdim16 + 16 * ct + l16] = acc[r];
         }
     }
-#undef CIE_BLOCKS_FETCH
-#pragma unroll
-    for (int u = 0; u < TPW; ++u)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int row = 16 * (wave * TPW + u) + 4 * g + r;
-            if (col_ok && row < dim) mem[static_cast<size_t>(row) * vdim] = S[u][r];
+}
+
+// One thread per number of a head's memory (rows and columns padded as `sums` has them): over the sequence's blocks in
+// order, the block's place gets the memory in front of the block, and the memory moves on by the block's sum.
+__global__ void __launch_bounds__(256)
+retention_scan_kernel(const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ seq_slot,
+                      const int* __restrict__ q_start_loc, float* __restrict__ sums, int heads, int dim, int vdim,
+                      int padded, int vdim16) {
+    const int seq = blockIdx.x / heads;
+    const int head = blockIdx.x - seq * heads;
+    const int e = blockIdx.y * blockDim.x + threadIdx.x;
+    if (e >= padded * vdim16) return;
+    const int first = q_start_loc[seq];
+    const int count = q_start_loc[seq + 1] - first;
+    if (count <= 0) return;
+    const int row = e / vdim16;
+    const int col = e - row * vdim16;
+    const bool real = row < dim && col < vdim;
+    float* mem = state + ((static_cast<size_t>(seq_slot[seq]) * heads + head) * dim + row) * vdim + col;
+    float S = real ? *mem : 0.f;
+    const int blocks = (count + kBlockTokens - 1) / kBlockTokens;
+    const float fade = decay[head];
+    float whole = 1.0f, rest = 1.0f;
+    for (int n = 0; n < kBlockTokens; ++n) whole *= fade;
+    for (int n = 0; n < count - (blocks - 1) * kBlockTokens; ++n) rest *= fade;
+    const size_t step = static_cast<size_t>(heads) * padded * vdim16;
+    float* at = sums + (static_cast<size_t>(first / kBlockTokens + seq) * heads + head) * padded * vdim16 + e;
+    float add = at[0];
+    for (int b = 0; b < blocks; ++b) {
+        const float next = at[static_cast<size_t>(min(b + 1, blocks - 1)) * step];  // (asked for before this block's place is written)
+        at[static_cast<size_t>(b) * step] = S;
+        S = (b == blocks - 1 ? rest : whole) * S + add;
+        add = next;
+    }
+    if (real) *mem = S;
+}
+
+__global__ void __launch_bounds__(256)
+retention_block_reads_kernel(const float* __restrict__ turned, const float* __restrict__ decay,
+                             const int* __restrict__ q_start_loc, const float* __restrict__ sums, float* __restrict__ raw,
+                             int heads, int vdim, int padded, int vdim16) {
+    const int seq = blockIdx.x / heads;
+    const int head = blockIdx.x - seq * heads;
+    const int first = q_start_loc[seq];
+    const int count = q_start_loc[seq + 1] - first;
+    const int c0 = blockIdx.y * kBlockTokens;
+    if (c0 >= count) return;
+    const int cn = min(kBlockTokens, count - c0);
+    const int panel0 = blockIdx.z * kPanelCols;
+    const int col_tiles = min(kPanelCols, vdim16 - panel0) / 16;
+    const int stride = padded + 4;
+    extern __shared__ float4 lds4[];
+    float* q_s = reinterpret_cast<float*>(lds4);          // [32][stride]
+    float* pw = q_s + kBlockTokens * stride;             // [33]
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int l16 = lane % 16;
+    const int g = lane / 16;
+    const int tiles = padded / 16;
+    decay_table(pw, decay[head]);
+    stage_rows(q_s, stride, turned, first + c0, cn, heads, head, padded, 0);
+    __syncthreads();
+    const int place = first / kBlockTokens + seq + blockIdx.y;
+    const float* before = sums + (static_cast<size_t>(place) * heads + head) * padded * vdim16 + panel0;
+    for (int ct = wave; ct < col_tiles; ct += 4) {
+        acc4_t o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+        const float* rows = before + static_cast<size_t>(4 * g) * vdim16 + 16 * ct + l16;
+#pragma unroll 2
+        for (int m = 0; m < tiles; ++m) {
+            const float4 a0 = *reinterpret_cast<const float4*>(q_s + l16 * stride + 16 * m + 4 * g);
+            const float4 a1 = *reinterpret_cast<const float4*>(q_s + (16 + l16) * stride + 16 * m + 4 * g);
+            const float* s = rows + static_cast<size_t>(16 * m) * vdim16;
+            const float b0 = s[0], b1 = s[vdim16], b2 = s[2 * vdim16], b3 = s[3 * vdim16];
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.x, b0, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.x, b0, o1, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.y, b1, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.y, b1, o1, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.z, b2, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.z, b2, o1, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.w, b3, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.w, b3, o1, 0, 0, 0);
         }
+        const int col = panel0 + 16 * ct + l16;
+        if (col < vdim) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * g + r;
+                float* dst = raw + static_cast<size_t>(first + c0) * heads * vdim + head * vdim + col;
+                if (i < cn) dst[static_cast<size_t>(i) * heads * vdim] = o0[r] * pw[i + 1];
+                if (16 + i < cn) dst[static_cast<size_t>(16 + i) * heads * vdim] = o1[r] * pw[16 + i + 1];
+            }
+        }
+    }
 }
 
 // o / sqrt(mean(o^2) + eps) [* weight] * gate: one wave per (token, run of `span` heads).  The mean runs over the
@@ -650,14 +662,15 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
                           const int* seq_slot, const int* positions, const int* q_start_loc, float* turned, float* raw,
                           void* out, int tokens, int sequences, int heads, int dim, int vdim, int rows_per_thread,
                           int groups, int parts, int slice, int chunk, float eps, float key_scale, int act,
-                          int norm_span, const float* norm_weight, int gate_act, int blocks) {
+                          int norm_span, const float* norm_weight, int gate_act, int blocks, float* sums) {
     if (act < 0 || act > 1 || norm_span < 1 || heads % norm_span || gate_act < 0 || gate_act > 1) return CIE_BAD_ARGUMENT;
     if (blocks) {
-        // the walk in blocks on the matrix cores: one plane of o, queries and keys padded to whole tiles of 16
+        // the walk in blocks on the matrix cores: two planes of o, queries and keys padded to whole tiles of 16
+        if (!sums) return CIE_BAD_ARGUMENT;
         groups = 1;
         rows_per_thread = 16;
         parts = (dim + 15) / 16;
-        slice = vdim < kBlockCols ? vdim : kBlockCols;
+        slice = vdim < 16 ? vdim : 16;
         chunk = 1;
     }
     if (sequences < 0 || tokens < 0 || heads <= 0 || heads > 65535 || dim <= 0 || vdim <= 0 || groups <= 0 || chunk <= 0 ||
@@ -675,10 +688,14 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
                     static_cast<long>(chunk) * 2 * rows / 4 > static_cast<long>(kFetchPieces) * threads ||
                     static_cast<long>(chunk) * slice > static_cast<long>(kFetchValues) * threads))
         return CIE_BAD_ARGUMENT;
-    const size_t blocks_lds = sizeof(float) * (2 * static_cast<size_t>(kBlockTokens) * (padded + 4) + kBlockTokens * kBlockCols +
-                                               kBlockTokens * kScoreStride + 4 * kBlockTokens * kBlockCols + 36);
-    const int value_slices = (vdim + kBlockCols - 1) / kBlockCols;
-    if (blocks && (padded > 256 || blocks_lds > 64 * 1024 || value_slices > 65535 ||
+    const int vdim16 = (vdim + 15) / 16 * 16;
+    const int panels = (vdim16 + kPanelCols - 1) / kPanelCols;
+    const int most_blocks = (tokens + kBlockTokens - 1) / kBlockTokens;  // (of one sequence: the grid's second size)
+    const size_t sums_lds = sizeof(float) * (2 * static_cast<size_t>(kBlockTokens) * (padded + 4) +
+                                             kBlockTokens * panel_stride(vdim16 < kPanelCols ? vdim16 : kPanelCols) +
+                                             kBlockTokens * kScoreStride + 36);
+    const size_t reads_lds = sizeof(float) * (static_cast<size_t>(kBlockTokens) * (padded + 4) + 36);
+    if (blocks && (sums_lds > 64 * 1024 || most_blocks > 65535 || panels > 65535 ||
                    static_cast<long>(sequences) * heads > 0x7fffffffL))
         return CIE_BAD_ARGUMENT;
     if (sequences == 0 || tokens == 0) return CIE_OK;
@@ -698,25 +715,26 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
     const long plane = static_cast<long>(tokens) * heads * vdim;
     int code = CIE_BAD_ARGUMENT;
     if (blocks) {
-        // (the workgroups of one head follow each other at a distance of `sequences * heads`: where that is a multiple
-        // of eight they share an XCD, and its L2 holds the head's queries and keys for all of them)
-        const dim3 block_grid(sequences * heads, value_slices);
-#define CIE_BLOCKS(T, TPW)                                                                                            \
-    retention_blocks_kernel<T, TPW><<<block_grid, 256, blocks_lds, s>>>(static_cast<const T*>(proj), ldp, v_off, turned,   \
-                                                                          decay, state, seq_slot, q_start_loc, raw, heads, \
-                                                                          dim, vdim, padded, act)
-        if (dtype == CIE_F32) {
-            if (padded <= 64) CIE_BLOCKS(float, 1);
-            else if (padded <= 128) CIE_BLOCKS(float, 2);
-            else CIE_BLOCKS(float, 4);
-        } else {
-            if (padded <= 64) CIE_BLOCKS(bf16_t, 1);
-            else if (padded <= 128) CIE_BLOCKS(bf16_t, 2);
-            else CIE_BLOCKS(bf16_t, 4);
-        }
-#undef CIE_BLOCKS
+        const dim3 block_grid(sequences * heads, most_blocks, panels);
+        if (dtype == CIE_F32)
+            retention_block_sums_kernel<float><<<block_grid, 256, sums_lds, s>>>(
+                static_cast<const float*>(proj), ldp, v_off, turned, decay, q_start_loc, raw, sums, heads, vdim, padded,
+                vdim16, act);
+        else
+            retention_block_sums_kernel<bf16_t><<<block_grid, 256, sums_lds, s>>>(
+                static_cast<const bf16_t*>(proj), ldp, v_off, turned, decay, q_start_loc, raw, sums, heads, vdim, padded,
+                vdim16, act);
         code = cie_after_launch();
-        parts = 1;
+        if (code != CIE_OK) return code;
+        const dim3 scan_grid(sequences * heads, (padded * vdim16 + 255) / 256);
+        retention_scan_kernel<<<scan_grid, 256, 0, s>>>(decay, state, seq_slot, q_start_loc, sums, heads, dim, vdim, padded,
+                                                       vdim16);
+        code = cie_after_launch();
+        if (code != CIE_OK) return code;
+        retention_block_reads_kernel<<<block_grid, 256, reads_lds, s>>>(turned, decay, q_start_loc, sums, raw + plane, heads,
+                                                                         vdim, padded, vdim16);
+        code = cie_after_launch();
+        parts = 2;
     } else {
         dim3 grid(sequences, heads, slices * parts);
 #define CIE_RETENTION(T, DS)                                                                                         \

@@ -933,7 +933,8 @@ RETENTION_LDS_FLOATS = 15 * 1024
 RETENTION_ACTIVATIONS = {None: 0, "silu": 1}   # what queries, keys and values pass through on their way in
 RETENTION_GATES = {"silu": 0, "sigmoid": 1}    # the function of the gate columns that multiplies the read-out
 RETENTION_BLOCKS_FROM = 16       # tokens a sequence (on average) from which the walk goes in blocks on the matrix cores
-RETENTION_BLOCKS_MAX_DIM = 192   # ... for heads whose queries and keys of a block fit the LDS
+RETENTION_BLOCKS_MAX_DIM = 160   # ... for heads whose queries, keys and values of a block fit the LDS
+RETENTION_BLOCKS_MAX_BYTES = 2 << 30  # ... and whose blocks' sums fit this much scratch memory
 
 
 def plan_retention(dim: int, vdim: int, units: int = 1) -> tuple[int, int, int, int, int]:
@@ -1008,12 +1009,18 @@ def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optio
             raise ValueError(f"{name} has {meta.shape[0]} entries, {least} are needed")
     rows, groups, parts, piece, chunk = plan_retention(dim, vdim, max(1, sequences * heads))
     # sequences that bring many tokens (prompts' portions) walk in blocks of 32 tokens on the matrix cores, float32
-    # operands and sums; steps of few tokens a sequence walk token by token.  (The same sums in another order.)
-    blocks = tokens >= RETENTION_BLOCKS_FROM * max(sequences, 1) and dim <= RETENTION_BLOCKS_MAX_DIM
+    # operands and sums, every block's own sums at once and only the memory itself in order; steps of few tokens a
+    # sequence walk token by token.  (The same sums in another order.)
+    padded, vdim16 = -(-dim // 16) * 16, -(-vdim // 16) * 16
+    places = tokens // 32 + sequences + 1
+    blocks = (tokens >= RETENTION_BLOCKS_FROM * max(sequences, 1) and dim <= RETENTION_BLOCKS_MAX_DIM
+              and places * heads * padded * vdim16 * 4 <= RETENTION_BLOCKS_MAX_BYTES)
+    sums = None
     if blocks:
-        rows, groups, parts = 16, 1, -(-dim // 16)
+        rows, groups, parts = 16, 1, padded // 16
+        sums = torch.empty((places, heads, padded, vdim16), dtype=torch.float32, device=proj.device)
     turned = torch.empty((tokens, heads, 2, parts * groups * rows), dtype=torch.float32, device=proj.device)
-    raw = torch.empty((1 if blocks else parts, tokens, heads * vdim), dtype=torch.float32, device=proj.device)
+    raw = torch.empty((2 if blocks else parts, tokens, heads * vdim), dtype=torch.float32, device=proj.device)
     out = torch.empty((tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
     ldp = proj.stride(0) if tokens > 1 else max(proj.stride(0), proj.shape[1])
     _run("cie_retention", load_library().cie_retention(
@@ -1022,7 +1029,7 @@ def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optio
         _ptr(positions), _ptr(q_start_loc), _ptr(turned), _ptr(raw), _ptr(out), _i(tokens), _i(sequences), _i(heads), _i(dim), _i(vdim),
         _i(rows), _i(groups), _i(parts), _i(piece), _i(chunk), _f(eps), _f(key_scale),
         _i(RETENTION_ACTIVATIONS[activation]), _i(norm_span), _ptr(norm_weight), _i(RETENTION_GATES[gate]),
-        _i(1 if blocks else 0)))
+        _i(1 if blocks else 0), _ptr(sums)))
     return out
 
 

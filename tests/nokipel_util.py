@@ -62,7 +62,7 @@ SMALL_B = {
     "layers": [
         {"type": "attention",
          "mixer": {"heads": 5, "kv_heads": 1, "dim": 12, "vdim": 20, "scale": 0.4, "mask": {"size": 64},
-                   "rot": {"base": 250000.0, "dims": 4}},
+                   "rot": {"base": 10000.0, "dims": 4}},
          "mlp": {"kind": "moe", "router": {"experts": 10, "identity": 5, "top": 4, "scale": 2.0, "groups": {"count": 5, "keep": 2}},
                  "expert": {"ff": 30}, "shared": {"ff": 22}}},
         {"type": "lightning", "mixer": {"heads": 5, "dim": 8, "vdim": 16, "decay": [0.25, 0.5, 0.75, 0.875, 0.999]},
