@@ -29,8 +29,10 @@ __device__ __forceinline__ float gelu_tanh(float z) {
 
 // ---------------------------------------------------------------------------------------------- retention
 // Three kernels.  (a) Every token's queries and keys, turned by its position, the keys scaled, as float32 rows padded
-// with zeros to `padded` numbers per head: [tokens, heads, 2, padded].  (b) The walk over the tokens, below.  (c) The
-// head's norm and the gate, which need all value columns of a head.
+// with zeros to `padded` numbers per head: [tokens, heads, 2, padded] (what passes through an activation on its way in
+// does so here).  (b) The walk over the tokens, below, token by token for steps of few tokens a sequence, or (b') in
+// blocks on the matrix cores for prompts' portions.  (c) The norm over a head's or over several heads' read-outs, the
+// norm's weight and the gate, which need all value columns of the heads that share a root mean square.
 //
 // (b) A column of the memory never meets another column, and o_t is a sum over the memory's rows, so one workgroup
 // takes (sequence, head, slice of up to 64 value columns, part of the rows) and the parts' shares of o_t are added

@@ -978,7 +978,10 @@ def retention(proj: torch.Tensor, offsets: tuple[int, int, int, int], cos: Optio
     must reach ``longest_position``.  ``activation="silu"``: queries, keys and values pass through silu on their way
     in.  The read-out is divided by its root mean square over runs of ``norm_span`` heads (1: each head alone;
     ``heads``: the token's whole row), multiplied by ``norm_weight`` (float32 [heads * vdim]) where given, and by
-    ``silu`` or ``sigmoid`` (``gate``) of the gate columns.  Returns [T, heads * vdim] in ``proj``'s type."""
+    ``silu`` or ``sigmoid`` (``gate``) of the gate columns.  Steps of ``RETENTION_BLOCKS_FROM`` tokens a sequence and more
+    walk in blocks of 32 tokens on the matrix cores in float32 (heads of up to ``RETENTION_BLOCKS_MAX_DIM`` numbers a key,
+    scratch of up to ``RETENTION_BLOCKS_MAX_BYTES``), others token by token: the same sums in another order.
+    Returns [T, heads * vdim] in ``proj``'s type."""
     if activation not in RETENTION_ACTIVATIONS or gate not in RETENTION_GATES:
         raise ValueError(f"activation is one of {list(RETENTION_ACTIVATIONS)}, gate one of {list(RETENTION_GATES)}")
     if norm_span < 1 or heads % norm_span:

@@ -83,6 +83,9 @@ MECHANISMS = {
                                "mixer": {"heads": 2, "dim": 128, "vdim": 128, "decay": [0.9375, 0.99951171875]}},
     "lightning_long_keys": {"type": "lightning", "mlp": None,
                             "mixer": {"heads": 1, "dim": 160, "vdim": 24, "decay": [0.984375]}},
+    # keys too long for the walk by blocks: prompts walk token by token
+    "lightning_keys_beyond_the_blocks": {"type": "lightning", "mlp": None,
+                                         "mixer": {"heads": 2, "dim": 168, "vdim": 16, "decay": [0.9375, 0.9990234375]}},
     # rows of all heads' read-outs wider than one wave norms: 1,080 and 2,176 numbers
     "lightning_wide_rows": {"type": "lightning", "mlp": None,
                             "mixer": {"heads": 9, "dim": 4, "vdim": 120, "decay": [0.5 + 0.055 * h for h in range(9)]}},
