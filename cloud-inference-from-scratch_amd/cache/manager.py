@@ -47,19 +47,33 @@ class PagedKV:
     ``head_dim`` numbers and, if ``values``, a value of ``value_dim`` numbers
     (``None``: as wide as the key).  ``values=False`` is a cache of one vector
     per token and head (a latent that keys and values are both made from, or
-    keys alone).  With a ``window`` only that many latest tokens are read."""
+    keys alone).  With a ``window`` only that many latest tokens are read, and beside them the first
+    ``keep_first`` tokens of the sequence, whose pages stay when the window has passed them."""
 
     kv_heads: int
     head_dim: int
     window: int | None = None
     values: bool = True
     value_dim: int | None = None
+    keep_first: int = 0
 
     def __post_init__(self) -> None:
         if self.kv_heads < 1 or self.head_dim < 1:
             raise ValueError("a paged cache needs at least one head of at least one number")
         if self.value_dim is not None and (not self.values or self.value_dim < 1):
             raise ValueError("value_dim needs values=True and a positive width")
+        if self.keep_first < 0:
+            raise ValueError("keep_first is a count of tokens")
+
+    def joined(self, other: "PagedKV") -> "PagedKV":
+        """The need of a unit that ``other`` reads as well: what either reader still sees is kept."""
+        same = (self.kv_heads, self.head_dim, self.values, self.value_dim) == (
+            other.kv_heads, other.head_dim, other.values, other.value_dim)
+        if not same:
+            raise ValueError(f"{other} cannot read the cache unit of {self}: the heads differ")
+        window = None if self.window is None or other.window is None else max(self.window, other.window)
+        keep = 0 if window is None else max(self.keep_first, other.keep_first)
+        return PagedKV(self.kv_heads, self.head_dim, window, self.values, self.value_dim, keep)
 
     @property
     def value_width(self) -> int:
@@ -194,7 +208,7 @@ class CacheManager:
                 if spec not in by_spec:
                     pages, per_request = full_pages, None
                     if spec.window is not None:
-                        per_request = -(-(spec.window + prefill_chunk) // page_size) + 1
+                        per_request = -(-(spec.window + prefill_chunk) // page_size) + 1 + -(-spec.keep_first // page_size)
                         pages = min(full_pages, max_running * per_request)
                     by_spec[spec] = len(self.groups)
                     self.groups.append(_Group(spec, [], pages, page_size, per_request))
@@ -268,7 +282,8 @@ class CacheManager:
             if group.most_per_request is not None:
                 # the pages below the window's reach from where the request stands are never asked for again
                 # (a request that decodes behind a long prompt holds its window's pages and needs one more at most)
-                passed = max(0, held_tokens + 1 - group.spec.window) // self.page_size
+                kept = min(-(-group.spec.keep_first // self.page_size), pages)
+                passed = max(0, max(0, held_tokens + 1 - group.spec.window) // self.page_size - kept)
                 pages = min(pages - passed, group.most_per_request)
             table = group.tables.get(request_id, ())
             most = max(most, pages - sum(1 for page in table if page >= 0))
@@ -360,7 +375,8 @@ class CacheManager:
                 # the next query sits at position >= length and sees keys >= length + 1 - window
                 first_needed = max(0, self._length[request_id] + 1 - window)
                 table = group.tables[request_id]
-                passed = [i for i in range(min(first_needed // self.page_size, len(table))) if table[i] >= 0]
+                kept = -(-group.spec.keep_first // self.page_size)  # pages that hold some of the kept first tokens
+                passed = [i for i in range(kept, min(first_needed // self.page_size, len(table))) if table[i] >= 0]
                 if passed:
                     group.allocator.free([table[i] for i in passed], request_id)
                     for i in passed:

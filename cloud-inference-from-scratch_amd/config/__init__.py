@@ -3,6 +3,7 @@ from .givizen import GivizenConfig
 from .nokipel import NokipelConfig
 from .polosun import PolosunConfig
 from .qwen2 import Qwen2Config
+from .senuvik import SenuvikConfig
 from .registry import (
     ARCHITECTURES,
     Architecture,
@@ -18,9 +19,10 @@ register_architecture("Qwen2ForCausalLM", Qwen2Config, model_type="qwen2")
 register_architecture("Polosun", PolosunConfig)
 register_architecture("Givizen", GivizenConfig)
 register_architecture("Nokipel", NokipelConfig)
+register_architecture("Senuvik", SenuvikConfig)
 
 __all__ = [
     "ARCHITECTURES", "Architecture", "ConfigError", "EngineConfig", "GivizenConfig", "LayerCall", "LayerSpec",
-    "ModelSpec", "NokipelConfig", "PartSpec", "PolosunConfig", "Qwen2Config", "architecture_of", "build_engine_config",
+    "ModelSpec", "NokipelConfig", "PartSpec", "PolosunConfig", "Qwen2Config", "SenuvikConfig", "architecture_of", "build_engine_config",
     "canonical_dtype", "config_from_dict", "load_config", "register_architecture",
 ]

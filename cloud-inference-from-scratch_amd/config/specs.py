@@ -42,7 +42,8 @@ class LayerSpec:
     ``names`` maps the block's part roles (``norm1``, ``mixer``, ``norm2``,
     ``feed_forward``) to the sub-prefix of the checkpoint's tensor names.
     ``options`` are the arrangement's own constants (a factor on the branches, the layer's depth), which
-    the block class reads.
+    the block class reads.  ``norm1_out`` and ``norm2_out`` are the norms on the sublayers' outputs of an arrangement
+    that has norms on both sides of a sublayer.
     """
 
     mixer: PartSpec
@@ -52,6 +53,8 @@ class LayerSpec:
     block: str = "pre_norm"
     names: tuple[tuple[str, str], ...] = ()
     options: tuple[tuple[str, Any], ...] = ()
+    norm1_out: PartSpec | None = None
+    norm2_out: PartSpec | None = None
 
     def option(self, name: str, default: Any = None) -> Any:
         return dict(self.options).get(name, default)

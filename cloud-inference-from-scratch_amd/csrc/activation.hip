@@ -80,27 +80,27 @@ CIE_API int cie_silu_mul(void* stream, int dtype, const void* gate_up, void* out
 // The gated unit with bounded inputs (activation_forms.h) over rows [tokens, 2 * intermediate], gate half first.
 template <typename T>
 __global__ void clamped_glu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int intermediate, float limit,
-                                   float alpha, float offset) {
+                                   float alpha, float offset, float cubic) {
     const int token = blockIdx.x;
     const int i = blockIdx.y * blockDim.x + threadIdx.x;
     if (i >= intermediate) return;
     const T* row = gate_up + static_cast<size_t>(token) * 2 * intermediate;
     out[static_cast<size_t>(token) * intermediate + i] =
-        from_float<T>(clamped_glu(to_float(row[i]), to_float(row[intermediate + i]), limit, alpha, offset));
+        from_float<T>(clamped_glu(to_float(row[i]), to_float(row[intermediate + i]), limit, alpha, offset, cubic));
 }
 
 CIE_API int cie_clamped_glu(void* stream, int dtype, const void* gate_up, void* out, int tokens, int intermediate,
-                            float limit, float alpha, float offset) {
+                            float limit, float alpha, float offset, float cubic) {
     if (tokens < 0 || intermediate <= 0 || (intermediate + 255) / 256 > 65535 || !(limit > 0.f)) return CIE_BAD_ARGUMENT;
     if (tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     dim3 grid(tokens, (intermediate + 255) / 256);
     if (dtype == CIE_F32)
         clamped_glu_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gate_up), static_cast<float*>(out),
-                                                      intermediate, limit, alpha, offset);
+                                                      intermediate, limit, alpha, offset, cubic);
     else if (dtype == CIE_BF16)
         clamped_glu_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(gate_up), static_cast<bf16_t*>(out),
-                                                       intermediate, limit, alpha, offset);
+                                                       intermediate, limit, alpha, offset, cubic);
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();

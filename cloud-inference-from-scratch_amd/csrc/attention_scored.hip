@@ -5,6 +5,8 @@
 //   s_ij <- cap * tanh(s_ij / cap)                       cap > 0
 //   s_ij <- s_ij - slope[head] * (i - j)                 slopes given (a bias on the distance itself)
 //   j is seen by i when 0 <= i - j < window              window > 0 (else every j <= i)
+//   ... or, beside the window, when j < keep <= ...       keep > 0: the first `keep` keys of the sequence stay visible
+//                                                        to every later token, at their own positions
 //   ... or when j <= i and floor(i / chunk) = floor(j / chunk)   chunk > 0: chunks counted from position 0
 //   p_ij = exp(s_ij) / (sum_j exp(s_ij) + exp(sink[head]))   sinks given: one more term in the denominator, which
 //                                                        has no key and no value, no scale and no bias
@@ -15,7 +17,8 @@
 // the value sums and the gate are float32 in both storage types.
 //
 // `cie_heads_prepare` is what stands between the projection and this attention: a per-head RMS norm of queries
-// and keys (with a weight, without one, or none), the queries' factor that grows with the position,
+// and keys (with a weight, without one, or none; or one RMS norm over all query heads of a token together and one
+// over all its key heads, with a weight per number of the projection), the queries' factor that grows with the position,
 //   q <- q * (1 + coef * ln(floor((p + 1) / every) + 1)),
 // then a rotation of the first `rot` numbers of every query and key head by the position (pairs of neighbours or of
 // the two halves; cos and sin from float32 tables [positions, rot / 2]),
@@ -68,7 +71,17 @@ heads_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int
     const T* src = row + (is_q ? q_off : k_off) + head * dim;
     const float* weight = is_q ? q_weight : k_weight;
     float factor = 1.f;
-    if (norm_mode != 0) {
+    if (norm_mode == 3) {  // one root mean square over all heads of the projection; the weight has a number for each
+        const int all = (is_q ? q_heads : kv_heads) * dim;
+        const T* whole = row + (is_q ? q_off : k_off);
+        float sum_sq = 0.f;
+        for (int d = lane; d < all; d += kWave) {
+            const float x = to_float(whole[d]);
+            sum_sq += x * x;
+        }
+        factor = 1.0f / sqrtf(wave_sum(sum_sq) / static_cast<float>(all) + eps);
+        weight += head * dim;
+    } else if (norm_mode != 0) {
         float sum_sq = 0.f;
         for (int d = lane; d < dim; d += kWave) {
             const float x = to_float(src[d]);
@@ -76,6 +89,7 @@ heads_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int
         }
         factor = 1.0f / sqrtf(wave_sum(sum_sq) / static_cast<float>(dim) + eps);
     }
+    const bool weighted = norm_mode >= 2;
     float after = 1.f;  // the queries' factor of the position
     if (is_q && temp_every > 0)
         after = 1.0f + temp_coef * logf(static_cast<float>((pos + 1) / temp_every) + 1.0f);
@@ -88,7 +102,7 @@ heads_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int
         float x = 0.f;
         if (d < dim) {
             x = to_float(src[d]) * factor;
-            if (norm_mode == 2) x *= weight[d];
+            if (weighted) x *= weight[d];
             if (d < rot) {
                 // the pair (u, v) of the angle's index i turns to (u cos - v sin, v cos + u sin): neighbours
                 // (2i, 2i + 1) or the halves (i, i + rot / 2)
@@ -96,7 +110,7 @@ heads_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int
                 const bool is_u = neighbours ? !(d & 1) : d < half;
                 const int mate = neighbours ? d ^ 1 : (is_u ? d + half : d - half);
                 float y = to_float(src[mate]) * factor;
-                if (norm_mode == 2) y *= weight[mate];
+                if (weighted) y *= weight[mate];
                 const float c = cos_row[i], sn = sin_row[i];
                 x = is_u ? x * c - y * sn : x * c + y * sn;
             }
@@ -139,6 +153,7 @@ struct ScoreShape {
     const float* sinks;   // [q_heads] or null
     int window;           // <= 0: all keys
     int chunk;            // > 0: i sees j <= i only inside its own chunk, floor(i / chunk) == floor(j / chunk)
+    int keep;             // > 0 (with a window): keys 0 .. keep - 1 are seen from behind the window too
 };
 
 // The first key that the query at position `pos` sees.
@@ -179,9 +194,13 @@ scored_attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ k
     float m = -INFINITY;
     float l = 0.f;
     float acc[kMaxSlices] = {0.f, 0.f, 0.f, 0.f};
-    for (int base = lo + wave * kWave; base < len; base += 4 * kWave) {
-        const int key = base + lane;
-        const bool valid = key < len;
+    // the keys in the order they are walked: the kept first ones that lie in front of the window, then the window's
+    const int kept = (shape.window > 0 && shape.keep > 0) ? min(shape.keep, lo) : 0;
+    const int walk = kept + len - lo;
+    for (int base = wave * kWave; base < walk; base += 4 * kWave) {
+        const int at = base + lane;
+        const int key = at < kept ? at : at - kept + lo;
+        const bool valid = at < walk;
         float s = -INFINITY;
         uint32_t head_block = 0;
         uint32_t in_page = 0;
@@ -207,7 +226,7 @@ scored_attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ k
         l = l * alpha + wave_sum(p);
 #pragma unroll
         for (int i = 0; i < kMaxSlices; ++i) acc[i] *= alpha;
-        const int count = min(kWave, len - base);
+        const int count = min(kWave, walk - base);
         for (int j = 0; j < count; ++j) {
             const float pj = __shfl(p, j, kWave);
             const uint32_t block_j = __shfl(head_block, j, kWave);
@@ -332,12 +351,25 @@ __global__ void __launch_bounds__(64 * kScoredWaves, RT <= 2 ? 2 : 1) scored_att
     const int hi = start + q0 + n_tok;
     const int chunk = a.shape.chunk;
     const int lo = first_seen(start + q0, window, chunk);
+    // The blocks of keys are walked in an order of their own: with kept first keys that lie wholly in front of the
+    // window's first block, blocks 0 .. kept_span - 1 come first and the window's blocks follow them; a walked index at
+    // or beyond kept_span is `gap` keys short of the key it stands for.  Otherwise walked index and key are the same.
+    const int keep = (window > 0 && a.shape.keep > 0) ? a.shape.keep : 0;
     int range_begin = lo & ~(kKeysPerBlock - 1);
-    int range_end = hi;
+    int kept_span = 0, gap = 0;
+    if (keep > 0) {
+        const int kept_blocks = (min(keep, hi) + kKeysPerBlock - 1) & ~(kKeysPerBlock - 1);
+        if (kept_blocks < range_begin) {
+            kept_span = kept_blocks;
+            gap = range_begin - kept_blocks;
+        }
+        range_begin = 0;
+    }
+    int range_end = hi - gap;
     const int split = blockIdx.z;
     if (a.n_splits > 1) {
         range_begin += split * a.keys_per_split;
-        range_end = min(hi, range_begin + a.keys_per_split);
+        range_end = min(hi - gap, range_begin + a.keys_per_split);
     }
     const int first_pos = start + q0;            // position of the tile's first token (its window reaches back furthest)
     const int last_lo = first_seen(start + q0 + n_tok - 1, window, chunk);  // the first key the tile's last token sees
@@ -378,9 +410,13 @@ __global__ void __launch_bounds__(64 * kScoredWaves, RT <= 2 ? 2 : 1) scored_att
         for (int dt = 0; dt < ND; ++dt) o[rt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int kb = range_begin + wave * kKeysPerBlock; kb < range_end; kb += STEP) {
+    for (int at = range_begin + wave * kKeysPerBlock; at < range_end; at += STEP) {
+        const int kb = at < kept_span ? at : at + gap;  // the block's first key
+        const int block_end = range_end + (kb - at);    // where this share's keys end, counted in keys of this block's stretch
         // every row sees every key of the block: none lies behind the first token, none before the last one's window
-        const bool inner = kb + kKeysPerBlock - 1 <= first_pos && kb >= last_lo && kb + kKeysPerBlock <= range_end;
+        // (or all are kept first keys)
+        const bool inner = kb + kKeysPerBlock - 1 <= first_pos && (kb >= last_lo || kb + kKeysPerBlock <= keep) &&
+                           kb + kKeysPerBlock <= block_end;
         floatx4 s[RT][2];
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
@@ -423,7 +459,7 @@ __global__ void __launch_bounds__(64 * kScoredWaves, RT <= 2 ? 2 : 1) scored_att
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int key = kb + kt * 16 + g * 4 + i;
-                    const bool seen = inner || (key <= pos && key >= row_lo && key < range_end);
+                    const bool seen = inner || (key <= pos && (key >= row_lo || key < keep) && key < block_end);
                     float x = s[rt][kt][i] * scale;
                     if (cap > 0.f) x = cap * fast_tanh(x * inv_cap);
                     x = x * kLog2e - row_slope[rt] * static_cast<float>(pos - key);
@@ -651,8 +687,8 @@ CIE_API int cie_heads_prepare(void* stream, int dtype, const void* proj, int pro
                               const float* sin_table, int rot, int neighbours) {
     if (rot < 0 || rot % 2 || rot > dim || (rot > 0 && (!cos_table || !sin_table))) return CIE_BAD_ARGUMENT;
     if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || D < dim || DV < vdim ||
-        page_size <= 0 || (page_size & (page_size - 1)) || table_width <= 0 || norm_mode < 0 || norm_mode > 2 ||
-        (norm_mode == 2 && (!q_weight || !k_weight)) || (norm_mode != 0 && !(eps > 0.f)) || temp_every < 0 ||
+        page_size <= 0 || (page_size & (page_size - 1)) || table_width <= 0 || norm_mode < 0 || norm_mode > 3 ||
+        (norm_mode >= 2 && (!q_weight || (write_kv && !k_weight))) || (norm_mode != 0 && !(eps > 0.f)) || temp_every < 0 ||
         q_off < 0 || k_off < 0 || v_off < 0 || proj_stride <= 0)
         return CIE_BAD_ARGUMENT;
     if (tokens == 0) return CIE_OK;
@@ -684,7 +720,8 @@ CIE_API int cie_scored_attention_generic(void* stream, int dtype, const void* q,
                                          const int* positions, const int* seq_of_token, const int* seq_slot,
                                          const void* gate, int gate_stride, void* out, int tokens, int q_heads,
                                          int kv_heads, int D, int DV, int page_size, int window, float scale,
-                                         float softcap, const float* slopes, const float* sinks, int chunk) {
+                                         float softcap, const float* slopes, const float* sinks, int chunk,
+                                         int keep) {
     if (tokens < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || D <= 0 || D % 8 || DV <= 0 || DV % 8 ||
         D > kWave * kMaxSlices || DV > kWave * kMaxSlices || page_size <= 0 || table_width <= 0 || q_heads > 65535 ||
         (gate && gate_stride < q_heads))
@@ -693,8 +730,8 @@ CIE_API int cie_scored_attention_generic(void* stream, int dtype, const void* q,
     hipStream_t s = static_cast<hipStream_t>(stream);
     dim3 grid(tokens, q_heads);
     const size_t lds = (static_cast<size_t>(D) + 4 * DV) * sizeof(float);
-    if (chunk < 0 || (chunk > 0 && window > 0)) return CIE_BAD_ARGUMENT;
-    const ScoreShape shape{scale, softcap, slopes, sinks, window, chunk};
+    if (chunk < 0 || (chunk > 0 && window > 0) || keep < 0 || (keep > 0 && window <= 0)) return CIE_BAD_ARGUMENT;
+    const ScoreShape shape{scale, softcap, slopes, sinks, window, chunk, keep};
     if (dtype == CIE_F32)
         scored_attention_generic_kernel<float><<<grid, 256, lds, s>>>(
             static_cast<const float*>(q), static_cast<const float*>(k_pool), static_cast<const float*>(v_pool),
@@ -719,8 +756,8 @@ CIE_API int cie_scored_attention_mfma(void* stream, const void* q, const void* k
                                       int gate_stride, void* out, int q_heads, int kv_heads, int D, int DV,
                                       int page_size, int tokens_per_tile, int row_tiles, int window, float scale,
                                       float softcap, const float* slopes, const float* sinks, int n_splits,
-                                      int keys_per_split, float* part_o, float* part_ml, int chunk) {
-    if (chunk < 0 || (chunk > 0 && window > 0)) return CIE_BAD_ARGUMENT;
+                                      int keys_per_split, float* part_o, float* part_ml, int chunk, int keep) {
+    if (chunk < 0 || (chunk > 0 && window > 0) || keep < 0 || (keep > 0 && window <= 0)) return CIE_BAD_ARGUMENT;
     if (n_tiles < 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads || page_size < 4 ||
         (page_size & (page_size - 1)) || table_width <= 0 || tokens_per_tile < 1 || kv_heads > 65535 ||
         (tile_seq == nullptr) != (tile_q0 == nullptr) || (gate && gate_stride < q_heads))
@@ -755,7 +792,7 @@ CIE_API int cie_scored_attention_mfma(void* stream, const void* q, const void* k
     while ((1 << a.page_shift) < page_size) ++a.page_shift;
     a.tokens_per_tile = tokens_per_tile;
     a.n_tiles = n_tiles;
-    a.shape = ScoreShape{scale, softcap, slopes, sinks, window, chunk};
+    a.shape = ScoreShape{scale, softcap, slopes, sinks, window, chunk, keep};
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (D == 64 && DV == 64) return launch_scored<64, 64>(s, a, row_tiles);
     if (D == 128 && DV == 128) return launch_scored<128, 128>(s, a, row_tiles);

@@ -1,0 +1,386 @@
+// A memory of outer products per head, S [rows, cols] in float32, that every token fades, adds to and reads:
+//
+//     S_t[n, p] = decay_t[n] * S_(t-1)[n, p] + in_t[n] * val_t[p]
+//
+// read after the update (a state-space layer:  y_t[p] = sum_n out_t[n] S_t[n, p] + skip * val_t[p],  decay one number
+// per head and token, in/out shared by the heads of a group, val_t scaled by the token's step size for the update),
+// or before it, with a bonus on the token's own outer product (time mixing with a decay per row:
+// y_t[p] = sum_n out_t[n] (S_(t-1)[n, p] + bonus[n] in_t[n] val_t[p])).  Which of the two, the strides and which
+// operands exist are arguments, so that one walk serves both layers; all operands are float32 rows made by the
+// kernels in front of it.  The state lives in rows of a state tensor, one per request slot; a step reads what its
+// earlier steps left, runs its tokens in order and writes it back, so a sequence may be cut into steps anywhere.
+//
+// Beside the walk: the step sizes and decays of a state-space layer, the mixes of a token with the one before it
+// and the decays of a time-mixing layer, and the norm in groups over a walk's read-out with its gate.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
+__device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+
+struct WalkArgs {
+    const float* decay;   // decay[t * ld_decay + head * decay_head_stride + n * decay_row_stride]  (row stride 0: one per head)
+    long ld_decay;
+    int decay_head_stride;
+    int decay_row_stride;
+    const float* in;      // in[t * ld_in + (head / heads_per_group) * rows + n]
+    long ld_in;
+    const float* out;     // out[t * ld_out + (head / heads_per_group) * rows + n]
+    long ld_out;
+    int heads_per_group;
+    const float* bonus;   // [heads, rows] or null; with read_first only
+    const float* val;     // val[t * ld_val + head * cols + p]
+    long ld_val;
+    const float* val_scale;  // val_scale[t * ld_scale + head] or null: the update takes val * scale
+    long ld_scale;
+    const float* skip;    // [heads] or null: y += skip[head] * val
+    float* state;         // [slots, heads, rows, cols]
+    const int* seq_slot;
+    const int* q_start_loc;
+    float* y;             // [tokens, heads * cols]
+    int heads, rows, cols, slice, row_groups, chunk, read_first;
+};
+
+// One workgroup per (sequence, head, slice of columns).  Thread (column, row group g) keeps rows g * NS .. + NS - 1
+// of its column in registers.  Tokens go in chunks: the chunk's row operands are staged in LDS (a row group's numbers
+// NS + 4 floats apart from the next group's, so that the groups of a wave read different banks), every thread walks
+// the chunk's tokens in order, and the row groups' shares of y meet in LDS behind the chunk.  The order of every sum
+// depends on the sizes alone, never on what else the step holds.
+template <int NS>
+__global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
+    extern __shared__ float lds[];
+    const int seq = blockIdx.x;
+    const int head = blockIdx.y;
+    const int col0 = blockIdx.z * a.slice;
+    const int RG = a.row_groups;
+    const int pitch = NS + 4;
+    const int per_token = RG * pitch;
+    const bool per_row_decay = a.decay_row_stride != 0;
+    float* in_s = lds;                                   // [chunk][RG][pitch]
+    float* out_s = in_s + a.chunk * per_token;           // [chunk][RG][pitch]
+    float* dec_s = out_s + a.chunk * per_token;          // [chunk][RG][pitch] (a decay per row) or [chunk]
+    float* bon_s = dec_s + (per_row_decay ? a.chunk * per_token : a.chunk);  // [chunk][RG][pitch] with a bonus
+    float* val_s = bon_s + (a.bonus ? a.chunk * per_token : 0);              // [chunk][slice]
+    float* scl_s = val_s + a.chunk * a.slice;            // [chunk]
+    float* part_s = scl_s + a.chunk;                     // [chunk][RG][slice]
+
+    const int col = threadIdx.x % a.slice;
+    const int rg = threadIdx.x / a.slice;
+    const bool live = rg < RG && col0 + col < a.cols;
+    const int first = a.q_start_loc[seq];
+    const int count = a.q_start_loc[seq + 1] - first;
+    const int group = head / a.heads_per_group;
+    float* mine = a.state + ((static_cast<size_t>(a.seq_slot[seq]) * a.heads + head) * a.rows) * a.cols + col0 + col;
+    float S[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        const int n = rg * NS + i;
+        S[i] = (live && n < a.rows) ? mine[static_cast<size_t>(n) * a.cols] : 0.f;
+    }
+    const float skip = a.skip ? a.skip[head] : 0.f;
+    for (int from = 0; from < count; from += a.chunk) {
+        const int n_tok = min(a.chunk, count - from);
+        __syncthreads();  // (the chunk before has been summed)
+        for (int idx = threadIdx.x; idx < n_tok * RG * NS; idx += blockDim.x) {
+            const int t = idx / (RG * NS);
+            const int n = idx - t * (RG * NS);
+            const int at = t * per_token + (n / NS) * pitch + n % NS;
+            const size_t token = static_cast<size_t>(first + from + t);
+            const bool real = n < a.rows;
+            const float x = real ? a.in[token * a.ld_in + group * a.rows + n] : 0.f;
+            in_s[at] = x;
+            out_s[at] = real ? a.out[token * a.ld_out + group * a.rows + n] : 0.f;
+            if (per_row_decay)
+                dec_s[at] = real ? a.decay[token * a.ld_decay + head * a.decay_head_stride + n * a.decay_row_stride] : 0.f;
+            if (a.bonus) bon_s[at] = real ? a.bonus[head * a.rows + n] * x : 0.f;
+        }
+        for (int idx = threadIdx.x; idx < n_tok * a.slice; idx += blockDim.x) {
+            const int t = idx / a.slice;
+            const int c = idx - t * a.slice;
+            const size_t token = static_cast<size_t>(first + from + t);
+            val_s[idx] = col0 + c < a.cols ? a.val[token * a.ld_val + head * a.cols + col0 + c] : 0.f;
+        }
+        for (int t = threadIdx.x; t < n_tok; t += blockDim.x) {
+            const size_t token = static_cast<size_t>(first + from + t);
+            scl_s[t] = a.val_scale ? a.val_scale[token * a.ld_scale + head] : 1.f;
+            if (!per_row_decay) dec_s[t] = a.decay[token * a.ld_decay + head * a.decay_head_stride];
+        }
+        __syncthreads();
+        if (rg < RG) {
+            for (int t = 0; t < n_tok; ++t) {
+                const float* in_t = in_s + t * per_token + rg * pitch;
+                const float* out_t = out_s + t * per_token + rg * pitch;
+                const float raw = val_s[t * a.slice + col];
+                const float v = raw * scl_s[t];
+                float acc = 0.f;
+                if (a.read_first) {
+                    const float* dec_t = dec_s + t * per_token + rg * pitch;
+                    const float* bon_t = bon_s + t * per_token + rg * pitch;
+#pragma unroll
+                    for (int i = 0; i < NS; ++i) {
+                        const float bonus = a.bonus ? bon_t[i] : 0.f;
+                        acc = fmaf(out_t[i], fmaf(bonus, v, S[i]), acc);
+                        S[i] = fmaf(per_row_decay ? dec_t[i] : dec_s[t], S[i], in_t[i] * v);
+                    }
+                } else if (per_row_decay) {
+                    const float* dec_t = dec_s + t * per_token + rg * pitch;
+#pragma unroll
+                    for (int i = 0; i < NS; ++i) {
+                        S[i] = fmaf(dec_t[i], S[i], in_t[i] * v);
+                        acc = fmaf(out_t[i], S[i], acc);
+                    }
+                } else {
+                    const float d = dec_s[t];
+#pragma unroll
+                    for (int i = 0; i < NS; ++i) {
+                        S[i] = fmaf(d, S[i], in_t[i] * v);
+                        acc = fmaf(out_t[i], S[i], acc);
+                    }
+                }
+                part_s[(t * RG + rg) * a.slice + col] = acc;
+            }
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < n_tok * a.slice; idx += blockDim.x) {
+            const int t = idx / a.slice;
+            const int c = idx - t * a.slice;
+            if (col0 + c >= a.cols) continue;
+            float sum = 0.f;
+            for (int g = 0; g < RG; ++g) sum += part_s[(t * RG + g) * a.slice + c];
+            sum = fmaf(skip, val_s[idx], sum);
+            a.y[static_cast<size_t>(first + from + t) * a.heads * a.cols + head * a.cols + col0 + c] = sum;
+        }
+    }
+    if (!live) return;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        const int n = rg * NS + i;
+        if (n < a.rows) mine[static_cast<size_t>(n) * a.cols] = S[i];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------- state-space steps
+// Per (token, head): the step size dt = softplus(raw + bias) and the decay exp(-exp(a_log) * dt), float32.
+template <typename T>
+__global__ void __launch_bounds__(256)
+space_steps_kernel(const T* __restrict__ raw, long ld, const float* __restrict__ bias, const float* __restrict__ a_log,
+                   float* __restrict__ steps, float* __restrict__ decay, long count, int heads) {
+    const long idx = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= count) return;
+    const long token = idx / heads;
+    const int head = static_cast<int>(idx - token * heads);
+    const float dt = softplus_f(to_float(raw[token * ld + head]) + bias[head]);
+    steps[idx] = dt;
+    decay[idx] = expf(-expf(a_log[head]) * dt);
+}
+
+// ---------------------------------------------------------------------------------------------- token shift
+// mixes[s][t] = h_t + (h_(t-1) - h_t) * mu[s] for each of `n_mix` weight rows mu[s]; the token in front of a step's
+// first token comes from the state (zeros for a new sequence).  The state is moved on by `time_decay_kernel`, which
+// runs behind everything that reads it.
+template <typename T>
+__global__ void __launch_bounds__(256)
+shift_mix_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ before, const float* __restrict__ mu,
+                 const int* __restrict__ seq_of_token, const int* __restrict__ seq_slot,
+                 const int* __restrict__ q_start_loc, T* __restrict__ mixes, int tokens, int width, int n_mix) {
+    const int token = blockIdx.x;
+    const int seq = seq_of_token[token];
+    const bool first = token == q_start_loc[seq];
+    const T* row = h + static_cast<size_t>(token) * ldh;
+    const T* prev = h + static_cast<size_t>(token - 1) * ldh;
+    const float* kept = before + static_cast<size_t>(seq_slot[seq]) * width;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const float x = to_float(row[c]);
+        const float d = (first ? kept[c] : to_float(prev[c])) - x;
+        for (int s = 0; s < n_mix; ++s)
+            mixes[(static_cast<size_t>(s) * tokens + token) * width + c] =
+                from_float<T>(fmaf(d, mu[static_cast<size_t>(s) * width + c], x));
+    }
+}
+
+// w[t, c] = exp(-exp(w2[c, :] . tanh(low[t, :]) + w0[c])): the decay of every key channel from the low-rank
+// projection of its mix (float32 [tokens, rank]).  One workgroup per token; tanh(low) is staged in LDS.  Also moves
+// the token-shift state on: the step's last token of every sequence leaves its input row there.
+template <typename T>
+__global__ void __launch_bounds__(256)
+time_decay_kernel(const float* __restrict__ low, const T* __restrict__ w2, const float* __restrict__ w0,
+                  float* __restrict__ decay, int channels, int rank, const T* __restrict__ h, long ldh,
+                  float* __restrict__ before, const int* __restrict__ seq_of_token, const int* __restrict__ seq_slot,
+                  const int* __restrict__ q_start_loc, int width) {
+    extern __shared__ float bent[];
+    const int token = blockIdx.x;
+    for (int r = threadIdx.x; r < rank; r += blockDim.x) bent[r] = tanhf(low[static_cast<size_t>(token) * rank + r]);
+    __syncthreads();
+    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+        const T* row = w2 + static_cast<size_t>(c) * rank;
+        float sum = 0.f;
+        for (int r = 0; r < rank; ++r) sum = fmaf(to_float(row[r]), bent[r], sum);
+        decay[static_cast<size_t>(token) * channels + c] = expf(-expf(sum + w0[c]));
+    }
+    const int seq = seq_of_token[token];
+    if (token + 1 == q_start_loc[seq + 1]) {
+        float* kept = before + static_cast<size_t>(seq_slot[seq]) * width;
+        const T* row = h + static_cast<size_t>(token) * ldh;
+        for (int c = threadIdx.x; c < width; c += blockDim.x) kept[c] = to_float(row[c]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------- read-out norm
+// out[t] = norm(y[t] * silu(gate[t])) * weight      (gate_first: the gate comes before the norm)
+// out[t] = norm(y[t]) * weight * silu(gate[t])      (otherwise)
+// with the norm over `groups` equal consecutive parts of the row, each divided by sqrt(mean(part^2) + eps).  y is
+// float32 [tokens, width]; the gate a view of T rows `ldg` apart; everything inside is float32.  One workgroup per
+// token, a wave per group in turn, the row staged in LDS.
+template <typename T>
+__global__ void __launch_bounds__(1024)
+gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate, long ldg,
+                        const float* __restrict__ weight, T* __restrict__ out, int width, int groups, float eps,
+                        int gate_first) {
+    extern __shared__ float staged[];  // [width], then [groups]
+    float* inverse = staged + width;
+    const size_t token = blockIdx.x;
+    const float* row = y + token * width;
+    const T* g_row = gate ? gate + token * ldg : nullptr;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float x = row[c];
+        if (g_row && gate_first) x *= silu_f(to_float(g_row[c]));
+        staged[c] = x;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x % kWave;
+    const int waves = blockDim.x / kWave;
+    const int per = width / groups;
+    for (int g = threadIdx.x / kWave; g < groups; g += waves) {
+        float sum_sq = 0.f;
+        for (int c = lane; c < per; c += kWave) {
+            const float x = staged[g * per + c];
+            sum_sq += x * x;
+        }
+        sum_sq = wave_sum(sum_sq);
+        if (lane == 0) inverse[g] = 1.0f / sqrtf(sum_sq / static_cast<float>(per) + eps);
+    }
+    __syncthreads();
+    T* dst = out + token * width;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float x = staged[c] * inverse[c / per];
+        if (weight) x *= weight[c];
+        if (g_row && !gate_first) x *= silu_f(to_float(g_row[c]));
+        dst[c] = from_float<T>(x);
+    }
+}
+
+}  // namespace
+
+// The walk (see the head of this file).  `rows_per_thread` in {8, 16, 32, 64}; `row_groups * rows_per_thread >= rows`;
+// `slice` columns a workgroup, `slice * row_groups <= 512` threads; `chunk` tokens staged at once.
+CIE_API int cie_memory_walk(void* stream, const float* decay, long ld_decay, int decay_head_stride, int decay_row_stride,
+                            const float* in, long ld_in, const float* out, long ld_out, int heads_per_group,
+                            const float* bonus, const float* val, long ld_val, const float* val_scale, long ld_scale,
+                            const float* skip, float* state, const int* seq_slot, const int* q_start_loc, float* y,
+                            int sequences, int heads, int rows, int cols, int rows_per_thread, int row_groups, int slice,
+                            int chunk, int read_first) {
+    if (sequences < 0 || heads <= 0 || heads > 65535 || rows <= 0 || cols <= 0 || heads_per_group <= 0 ||
+        heads % heads_per_group || row_groups <= 0 || slice <= 0 || chunk <= 0 ||
+        static_cast<long>(rows_per_thread) * row_groups < rows || slice * row_groups > 512 || !decay || !in || !out ||
+        !val || !state || !y || (bonus && !read_first))
+        return CIE_BAD_ARGUMENT;
+    const int slices = (cols + slice - 1) / slice;
+    if (slices > 65535) return CIE_BAD_ARGUMENT;
+    const int per_token = row_groups * (rows_per_thread + 4);
+    const size_t floats = static_cast<size_t>(chunk) *
+                              (2 * per_token + (decay_row_stride ? per_token : 1) + (bonus ? per_token : 0) + slice + 1 +
+                               static_cast<size_t>(row_groups) * slice);
+    if (floats * sizeof(float) > 64 * 1024) return CIE_BAD_ARGUMENT;
+    if (sequences == 0) return CIE_OK;
+    WalkArgs a{decay, ld_decay, decay_head_stride, decay_row_stride, in, ld_in, out, ld_out, heads_per_group, bonus,
+               val, ld_val, val_scale, ld_scale, skip, state, seq_slot, q_start_loc, y, heads, rows, cols, slice,
+               row_groups, chunk, read_first};
+    const int threads = ((slice * row_groups + kWave - 1) / kWave) * kWave;
+    const dim3 grid(sequences, heads, slices);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t lds = floats * sizeof(float);
+    if (rows_per_thread == 8) memory_walk_kernel<8><<<grid, threads, lds, s>>>(a);
+    else if (rows_per_thread == 16) memory_walk_kernel<16><<<grid, threads, lds, s>>>(a);
+    else if (rows_per_thread == 32) memory_walk_kernel<32><<<grid, threads, lds, s>>>(a);
+    else if (rows_per_thread == 64) memory_walk_kernel<64><<<grid, threads, lds, s>>>(a);
+    else return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+CIE_API int cie_space_steps(void* stream, int dtype, const void* raw, long ld, const float* bias, const float* a_log,
+                            float* steps, float* decay, int tokens, int heads) {
+    if (tokens < 0 || heads <= 0 || ld < heads || !bias || !a_log || !steps || !decay) return CIE_BAD_ARGUMENT;
+    if (tokens == 0) return CIE_OK;
+    const long count = static_cast<long>(tokens) * heads;
+    const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == CIE_F32)
+        space_steps_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(raw), ld, bias, a_log, steps, decay, count, heads);
+    else if (dtype == CIE_BF16)
+        space_steps_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(raw), ld, bias, a_log, steps, decay, count, heads);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+CIE_API int cie_shift_mix(void* stream, int dtype, const void* h, long ldh, const float* before, const float* mu,
+                          const int* seq_of_token, const int* seq_slot, const int* q_start_loc, void* mixes, int tokens,
+                          int width, int n_mix) {
+    if (tokens < 0 || width <= 0 || n_mix <= 0 || ldh < width || !before || !mu) return CIE_BAD_ARGUMENT;
+    if (tokens == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (dtype == CIE_F32)
+        shift_mix_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(h), ldh, before, mu, seq_of_token, seq_slot,
+                                                      q_start_loc, static_cast<float*>(mixes), tokens, width, n_mix);
+    else if (dtype == CIE_BF16)
+        shift_mix_kernel<bf16_t><<<tokens, 256, 0, s>>>(static_cast<const bf16_t*>(h), ldh, before, mu, seq_of_token, seq_slot,
+                                                       q_start_loc, static_cast<bf16_t*>(mixes), tokens, width, n_mix);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+CIE_API int cie_time_decay(void* stream, int dtype, const float* low, const void* w2, const float* w0, float* decay,
+                           int tokens, int channels, int rank, const void* h, long ldh, float* before,
+                           const int* seq_of_token, const int* seq_slot, const int* q_start_loc, int width) {
+    if (tokens < 0 || channels <= 0 || rank <= 0 || rank > 8192 || width <= 0 || ldh < width || !low || !w2 || !w0 ||
+        !decay || !h || !before)
+        return CIE_BAD_ARGUMENT;
+    if (tokens == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t lds = static_cast<size_t>(rank) * sizeof(float);
+    if (dtype == CIE_F32)
+        time_decay_kernel<float><<<tokens, 256, lds, s>>>(low, static_cast<const float*>(w2), w0, decay, channels, rank,
+                                                         static_cast<const float*>(h), ldh, before, seq_of_token,
+                                                         seq_slot, q_start_loc, width);
+    else if (dtype == CIE_BF16)
+        time_decay_kernel<bf16_t><<<tokens, 256, lds, s>>>(low, static_cast<const bf16_t*>(w2), w0, decay, channels, rank,
+                                                          static_cast<const bf16_t*>(h), ldh, before, seq_of_token,
+                                                          seq_slot, q_start_loc, width);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+CIE_API int cie_gated_group_norm(void* stream, int dtype, const float* y, const void* gate, long ldg,
+                                 const float* weight, void* out, int tokens, int width, int groups, float eps,
+                                 int gate_first) {
+    if (tokens < 0 || width <= 0 || groups <= 0 || width % groups || !(eps > 0.f) || !y || !out ||
+        (gate && ldg < width) || (static_cast<size_t>(width) + groups) * sizeof(float) > 64 * 1024)
+        return CIE_BAD_ARGUMENT;
+    if (tokens == 0) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int threads = width >= 2048 ? 1024 : width >= 1024 ? 512 : 256;
+    const size_t lds = (static_cast<size_t>(width) + groups) * sizeof(float);
+    if (dtype == CIE_F32)
+        gated_group_norm_kernel<float><<<tokens, threads, lds, s>>>(y, static_cast<const float*>(gate), ldg, weight,
+                                                                 static_cast<float*>(out), width, groups, eps, gate_first);
+    else if (dtype == CIE_BF16)
+        gated_group_norm_kernel<bf16_t><<<tokens, threads, lds, s>>>(y, static_cast<const bf16_t*>(gate), ldg, weight,
+                                                                  static_cast<bf16_t*>(out), width, groups, eps, gate_first);
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}

@@ -149,25 +149,37 @@ CIE_API int cie_add_rmsnorm(void* stream, int dtype, int wdtype, float* residual
     return CIE_BAD_ARGUMENT;
 }
 
-// Norm on a branch's output, then the add:  y = branch[row] (+ the sum of `parts` float32 rows [tokens, parts, hidden]);
+// Norm on a branch's output, then the add:
+//   y = scale_a * branch[row] * sigmoid(branch_gate[row]) + scale_b * branch2[row]
+//       + sum_p part_weight[row, p] * parts[row, p, :]           (float32 rows [tokens, parts, hidden], in order)
 //   residual[row] += y / sqrt(mean(y^2) + eps) * weight
-// (the weight as it multiplies: a weight stored around zero comes here with the one added).  With `rows_out`
-// the new stream is also written in the activation type, for the products of the sublayer that reads it next.
-// Statistics, scaling and the sum are float32.  One workgroup per row, the row staged in LDS.
+// Every addend but one may be absent (no gate: 1; no part weights: 1).  The weight comes as it multiplies: a weight
+// stored around zero with the one added, a norm's weight times a scale per channel as their product.  With
+// `rows_out` the new stream is also written in the activation type, for the products of a sublayer that reads the
+// stream itself; with `next_weight` the RMS norm of the new stream under that weight is written to `normed_out`, for
+// the sublayer that reads a norm of it.  Statistics, scaling and the sums are float32.  One workgroup per row, the
+// row staged in LDS.
 template <typename B, typename T>
 __global__ void branch_norm_add_kernel(float* __restrict__ residual, const B* __restrict__ branch,
-                                       const float* __restrict__ parts, int n_parts,
+                                       const float* __restrict__ branch_gate, int gate_stride,
+                                       const B* __restrict__ branch2, float scale_a, float scale_b,
+                                       const float* __restrict__ parts, const float* __restrict__ part_weight, int n_parts,
                                        const float* __restrict__ weight, T* __restrict__ rows_out, int hidden,
-                                       float eps) {
+                                       float eps, const float* __restrict__ next_weight, T* __restrict__ normed_out) {
     extern __shared__ float staged[];
     __shared__ float scratch[16];
     const size_t row = blockIdx.x;
     const B* add = branch ? branch + row * hidden : nullptr;
+    const B* add2 = branch2 ? branch2 + row * hidden : nullptr;
+    const float open = (branch && branch_gate) ? scale_a / (1.0f + expf(-branch_gate[row * gate_stride])) : scale_a;
     const float* extra = parts ? parts + row * n_parts * hidden : nullptr;
+    const float* extra_w = (parts && part_weight) ? part_weight + row * n_parts : nullptr;
     float sum_sq = 0.f;
     for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
-        float y = add ? to_float(add[h]) : 0.f;
-        for (int p = 0; p < n_parts; ++p) y += extra[static_cast<size_t>(p) * hidden + h];
+        float y = add ? to_float(add[h]) * open : 0.f;
+        if (add2) y = fmaf(scale_b, to_float(add2[h]), y);
+        for (int p = 0; p < n_parts; ++p)
+            y = fmaf(extra_w ? extra_w[p] : 1.0f, extra[static_cast<size_t>(p) * hidden + h], y);
         staged[h] = y;
         sum_sq += y * y;
     }
@@ -175,34 +187,47 @@ __global__ void branch_norm_add_kernel(float* __restrict__ residual, const B* __
     const float inv = 1.0f / sqrtf(total / static_cast<float>(hidden) + eps);
     float* res = residual + row * hidden;
     T* dst = rows_out ? rows_out + row * hidden : nullptr;
+    float next_sq = 0.f;
     for (int h = threadIdx.x; h < hidden; h += blockDim.x) {
         const float x = res[h] + (staged[h] * inv) * weight[h];
         res[h] = x;
         if (dst) dst[h] = from_float<T>(x);
+        staged[h] = x;
+        next_sq += x * x;
     }
+    if (!next_weight) return;
+    const float next_total = block_sum(next_sq, scratch);
+    const float next_inv = 1.0f / sqrtf(next_total / static_cast<float>(hidden) + eps);
+    T* normed = normed_out + row * hidden;
+    for (int h = threadIdx.x; h < hidden; h += blockDim.x)
+        normed[h] = from_float<T>((staged[h] * next_inv) * next_weight[h]);
 }
 
-// bdtype: storage type of `branch` (ignored without one); dtype: type of rows_out.
+// bdtype: storage type of `branch` and `branch2` (ignored without them); dtype: type of rows_out and normed_out.
 CIE_API int cie_branch_norm_add(void* stream, int bdtype, int dtype, float* residual, const void* branch,
-                                const float* parts, int n_parts, const float* weight, void* rows_out, int tokens,
-                                int hidden, float eps) {
+                                const float* branch_gate, int gate_stride, const void* branch2, float scale_a,
+                                float scale_b, const float* parts, const float* part_weight, int n_parts,
+                                const float* weight, void* rows_out, int tokens, int hidden, float eps,
+                                const float* next_weight, void* normed_out) {
     if (tokens < 0 || hidden <= 0 || hidden * sizeof(float) > 64 * 1024 || !(eps > 0.f) || n_parts < 0 ||
-        (n_parts > 0 && !parts) || (!branch && n_parts == 0))
+        (n_parts > 0 && !parts) || (!branch && !branch2 && n_parts == 0) || gate_stride < 1 ||
+        (next_weight && !normed_out))
         return CIE_BAD_ARGUMENT;
     if (tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int threads = tokens <= 64 ? 1024 : 256;
     const size_t lds = hidden * sizeof(float);
     if (!parts) n_parts = 0;
-    if (dtype == CIE_F32 && (bdtype == CIE_F32 || !branch))
-        branch_norm_add_kernel<float, float><<<tokens, threads, lds, s>>>(
-            residual, static_cast<const float*>(branch), parts, n_parts, weight, static_cast<float*>(rows_out), hidden, eps);
-    else if (dtype == CIE_BF16 && bdtype == CIE_BF16)
-        branch_norm_add_kernel<bf16_t, bf16_t><<<tokens, threads, lds, s>>>(
-            residual, static_cast<const bf16_t*>(branch), parts, n_parts, weight, static_cast<bf16_t*>(rows_out), hidden, eps);
-    else if (dtype == CIE_BF16 && bdtype == CIE_F32)
-        branch_norm_add_kernel<float, bf16_t><<<tokens, threads, lds, s>>>(
-            residual, static_cast<const float*>(branch), parts, n_parts, weight, static_cast<bf16_t*>(rows_out), hidden, eps);
+    const bool any = branch || branch2;
+#define CIE_BRANCH_NORM(B, T)                                                                                        \
+    branch_norm_add_kernel<B, T><<<tokens, threads, lds, s>>>(                                                          \
+        residual, static_cast<const B*>(branch), branch_gate, gate_stride, static_cast<const B*>(branch2), scale_a,       \
+        scale_b, parts, part_weight, n_parts, weight, static_cast<T*>(rows_out), hidden, eps, next_weight,                \
+        static_cast<T*>(normed_out))
+    if (dtype == CIE_F32 && (bdtype == CIE_F32 || !any)) CIE_BRANCH_NORM(float, float);
+    else if (dtype == CIE_BF16 && bdtype == CIE_BF16) CIE_BRANCH_NORM(bf16_t, bf16_t);
+    else if (dtype == CIE_BF16 && (bdtype == CIE_F32 || !any)) CIE_BRANCH_NORM(float, bf16_t);
+#undef CIE_BRANCH_NORM
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();

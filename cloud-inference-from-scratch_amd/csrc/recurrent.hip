@@ -549,11 +549,12 @@ int launch_retention(hipStream_t s, dim3 grid, int threads, size_t lds, const vo
 }
 
 // ---------------------------------------------------------------------------------------------- convolution
-template <typename T>
+// (`act`: what the sum passes through, 0 nothing, 1 silu; O: the type it is stored in)
+template <typename T, typename O>
 __global__ void __launch_bounds__(256)
 causal_conv_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ taps_w, const T* __restrict__ bias,
                    const float* __restrict__ past, const int* __restrict__ seq_of_token, const int* __restrict__ seq_slot,
-                   const int* __restrict__ q_start_loc, T* __restrict__ out, int channels, int taps) {
+                   const int* __restrict__ q_start_loc, O* __restrict__ out, int channels, int taps, int act) {
     const int token = blockIdx.y;
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= channels) return;
@@ -569,7 +570,32 @@ causal_conv_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ taps
         acc = fmaf(to_float(taps_w[static_cast<size_t>(c) * taps + j]), in, acc);
     }
     if (bias) acc += to_float(bias[c]);
-    out[static_cast<size_t>(token) * channels + c] = from_float<T>(acc);
+    out[static_cast<size_t>(token) * channels + c] = from_float<O>(activated(acc, act));
+}
+
+// The convolution's state moved on by a step's inputs: of [what the state held, the step's inputs] the last
+// taps - 1 rows.  One thread per (sequence, channel); runs behind the convolution that still read the old rows.
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv_keep_kernel(const T* __restrict__ x, long ldx, float* __restrict__ past, const int* __restrict__ seq_slot,
+                 const int* __restrict__ q_start_loc, int channels, int taps) {
+    const int seq = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int keep_n = taps - 1;
+    if (c >= channels || keep_n <= 0) return;
+    const int first = q_start_loc[seq];
+    const int count = q_start_loc[seq + 1] - first;
+    float* before = past + static_cast<size_t>(seq_slot[seq]) * keep_n * channels;
+    float old[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) old[j] = j < keep_n ? before[static_cast<size_t>(j) * channels + c] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        if (j >= keep_n) break;
+        const int src = count + j;  // index into [old (keep_n), new (count)]
+        before[static_cast<size_t>(j) * channels + c] =
+            src < keep_n ? old[src < 16 ? src : 0] : to_float(x[static_cast<size_t>(first + src - keep_n) * ldx + c]);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------- gated recurrence
@@ -786,19 +812,40 @@ CIE_API int cie_retention(void* stream, int dtype, const void* proj, long ldp, i
 
 CIE_API int cie_causal_conv(void* stream, int dtype, const void* x, long ldx, const void* taps_w, const void* bias,
                             const float* past, const int* seq_of_token, const int* seq_slot, const int* q_start_loc,
-                            void* out, int tokens, int channels, int taps) {
-    if (tokens < 0 || tokens > 65535 * 1 || channels <= 0 || taps < 1 || taps > kMaxTaps || ldx < channels) return CIE_BAD_ARGUMENT;
+                            void* out, int tokens, int channels, int taps, int act, int out_f32) {
+    if (tokens < 0 || tokens > 65535 * 1 || channels <= 0 || taps < 1 || taps > kMaxTaps || ldx < channels || act < 0 ||
+        act > 1)
+        return CIE_BAD_ARGUMENT;
     if (tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     dim3 grid((channels + 255) / 256, tokens);
+#define CIE_CONV(T, O)                                                                                              \
+    causal_conv_kernel<T, O><<<grid, 256, 0, s>>>(static_cast<const T*>(x), ldx, static_cast<const T*>(taps_w),          \
+                                                  static_cast<const T*>(bias), past, seq_of_token, seq_slot,            \
+                                                  q_start_loc, static_cast<O*>(out), channels, taps, act)
+    if (dtype == CIE_F32) CIE_CONV(float, float);
+    else if (dtype == CIE_BF16 && out_f32) CIE_CONV(bf16_t, float);
+    else if (dtype == CIE_BF16) CIE_CONV(bf16_t, bf16_t);
+#undef CIE_CONV
+    else
+        return CIE_BAD_ARGUMENT;
+    return cie_after_launch();
+}
+
+// Moves the convolution's state on by the step's inputs (see conv_keep_kernel); call it behind cie_causal_conv.
+CIE_API int cie_conv_keep(void* stream, int dtype, const void* x, long ldx, float* past, const int* seq_slot,
+                          const int* q_start_loc, int sequences, int channels, int taps) {
+    if (sequences < 0 || sequences > 65535 || channels <= 0 || taps < 1 || taps > kMaxTaps || ldx < channels)
+        return CIE_BAD_ARGUMENT;
+    if (sequences == 0 || taps == 1) return CIE_OK;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    dim3 grid((channels + 255) / 256, sequences);
     if (dtype == CIE_F32)
-        causal_conv_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(x), ldx, static_cast<const float*>(taps_w),
-                                                      static_cast<const float*>(bias), past, seq_of_token, seq_slot,
-                                                      q_start_loc, static_cast<float*>(out), channels, taps);
+        conv_keep_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(x), ldx, past, seq_slot, q_start_loc,
+                                                     channels, taps);
     else if (dtype == CIE_BF16)
-        causal_conv_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(x), ldx, static_cast<const bf16_t*>(taps_w),
-                                                       static_cast<const bf16_t*>(bias), past, seq_of_token, seq_slot,
-                                                       q_start_loc, static_cast<bf16_t*>(out), channels, taps);
+        conv_keep_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(x), ldx, past, seq_slot, q_start_loc,
+                                                      channels, taps);
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();

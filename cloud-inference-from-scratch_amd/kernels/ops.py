@@ -1040,10 +1040,12 @@ MAX_CONV_TAPS = 16
 
 
 def causal_conv(x: torch.Tensor, taps_w: torch.Tensor, bias: Optional[torch.Tensor], past: torch.Tensor,
-                seq_of_token: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor) -> torch.Tensor:
-    """Per channel, ``out[t] = sum_j taps_w[c, j] * x[t - (taps - 1) + j] + bias[c]`` within each sequence; the inputs
-    before the step come from ``past`` (float32 [slots, max(taps - 1, 1), C], oldest first; zeros for a new
-    sequence).  x [T, C] (a view with unit inner stride), taps_w [C, taps]."""
+                seq_of_token: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor,
+                activation: Optional[str] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """Per channel, ``out[t] = act(sum_j taps_w[c, j] * x[t - (taps - 1) + j] + bias[c])`` within each sequence; the
+    inputs before the step come from ``past`` (float32 [slots, max(taps - 1, 1), C], oldest first; zeros for a new
+    sequence).  x [T, C] (a view with unit inner stride), taps_w [C, taps].  ``activation``: ``None`` or ``"silu"``;
+    ``out_dtype``: x's type, or float32."""
     if not (x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.dtype in _CODES):
         raise ValueError("x must be a float32 or bfloat16 GPU matrix with unit inner stride")
     tokens, channels = x.shape
@@ -1062,12 +1064,35 @@ def causal_conv(x: torch.Tensor, taps_w: torch.Tensor, bias: Optional[torch.Tens
         _gpu(name, meta, torch.int32, 1)
     if seq_of_token.shape[0] < tokens:
         raise ValueError("one sequence index per token")
-    out = torch.empty((tokens, channels), dtype=x.dtype, device=x.device)
+    if activation not in RETENTION_ACTIVATIONS or out_dtype not in (None, x.dtype, torch.float32):
+        raise ValueError(f"activation {activation!r} / out_dtype {out_dtype} are none the convolution has")
+    out = torch.empty((tokens, channels), dtype=out_dtype or x.dtype, device=x.device)
     ldx = x.stride(0) if tokens > 1 else max(x.stride(0), channels)
     _run("cie_causal_conv", load_library().cie_causal_conv(
         _stream(), _i(_code(x.dtype)), _ptr(x), ldx, _ptr(taps_w), _ptr(bias), _ptr(past), _ptr(seq_of_token),
-        _ptr(seq_slot), _ptr(q_start_loc), _ptr(out), _i(tokens), _i(channels), _i(taps)))
+        _ptr(seq_slot), _ptr(q_start_loc), _ptr(out), _i(tokens), _i(channels), _i(taps),
+        _i(RETENTION_ACTIVATIONS[activation]), _i(1 if out.dtype == torch.float32 else 0)))
     return out
+
+
+def conv_keep(x: torch.Tensor, past: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor, sequences: int,
+              taps: int) -> None:
+    """Moves a causal convolution's state on by a step's inputs ``x`` [T, C]: of what ``past`` (float32 [slots,
+    max(taps - 1, 1), C]) held and the step's rows, the last ``taps - 1`` stay.  Runs behind the convolution."""
+    if not (x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.dtype in _CODES):
+        raise ValueError("x must be a float32 or bfloat16 GPU matrix with unit inner stride")
+    tokens, channels = x.shape
+    _gpu("past", past, torch.float32, 3)
+    if tuple(past.shape[1:]) != (max(taps - 1, 1), channels) or not 1 <= taps <= MAX_CONV_TAPS:
+        raise ValueError(f"past {tuple(past.shape)} must be [slots, {max(taps - 1, 1)}, {channels}]")
+    for name, meta, least in (("seq_slot", seq_slot, sequences), ("q_start_loc", q_start_loc, sequences + 1)):
+        _gpu(name, meta, torch.int32, 1)
+        if meta.shape[0] < least:
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
+    ldx = x.stride(0) if tokens > 1 else max(x.stride(0), channels)
+    _run("cie_conv_keep", load_library().cie_conv_keep(_stream(), _i(_code(x.dtype)), _ptr(x), ldx, _ptr(past),
+                                                       _ptr(seq_slot), _ptr(q_start_loc), _i(sequences), _i(channels),
+                                                       _i(taps)))
 
 
 def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, gates: torch.Tensor, block_width: int,
@@ -1106,35 +1131,238 @@ def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, g
 
 
 # ---------------------------------------------------------------------------
+WALK_ROWS = (8, 16, 32, 64)   # rows of a memory that one thread of the walk keeps in registers
+WALK_MAX_ROWS = 1024
+WALK_LDS_BYTES = 48 * 1024
+
+
+def plan_memory_walk(rows: int, cols: int, per_row_decay: bool, bonus: bool, units: int = 1) -> tuple[int, int, int, int]:
+    """(rows per thread, row groups, columns per workgroup, tokens staged at once) of ``memory_walk`` for a memory
+    of ``rows`` x ``cols`` per head, of which ``units`` (sequences x heads) are walked at once.  Rows per thread and
+    row groups follow from ``rows`` alone (they fix the order of the read-out's sums); the columns are cut into more
+    workgroups while these are fewer than the compute units."""
+    if not (1 <= rows <= WALK_MAX_ROWS and cols >= 1):
+        raise ValueError(f"a memory of {rows} x {cols}: up to {WALK_MAX_ROWS} rows")
+    per_thread = 8 if rows <= 8 else 16 if rows <= 64 else 32 if rows <= 256 else 64
+    groups = -(-rows // per_thread)
+    widest = 1 << (min(cols, 64, 512 // groups) - 1).bit_length()  # (a power of two that holds the columns, at most 64)
+    widest = min(widest, 64)
+    while widest * groups > 512:
+        widest //= 2
+    slice_cols = widest
+    while slice_cols > 16 and units * -(-cols // slice_cols) < compute_units():
+        slice_cols //= 2
+    per_token = groups * (per_thread + 4)
+    floats = 2 * per_token + (per_token if per_row_decay else 1) + (per_token if bonus else 0) + slice_cols + 1 + groups * slice_cols
+    chunk = max(1, min(16, WALK_LDS_BYTES // (4 * floats)))
+    return per_thread, groups, slice_cols, chunk
+
+
+def memory_walk(decay: torch.Tensor, in_rows: torch.Tensor, out_rows: torch.Tensor, values: torch.Tensor,
+                state: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor, sequences: int, heads: int,
+                rows: int, cols: int, heads_per_group: int = 1, bonus: Optional[torch.Tensor] = None,
+                value_scale: Optional[torch.Tensor] = None, skip: Optional[torch.Tensor] = None,
+                read_first: bool = False) -> torch.Tensor:
+    """The walk of ``csrc/memory_walk.hip`` over a step's tokens: per head a float32 memory ``S`` [rows, cols] in
+    ``state`` [slots, heads, rows, cols], ``S <- decay * S + in (x) (value * value_scale)`` token by token, and the
+    read-out ``y = S^T out + skip * value`` behind the update, or (``read_first``) ``y = (S + (bonus * in) (x) value)^T
+    out`` in front of it.  All operands float32 views with unit inner stride: ``decay`` [T, heads] (one per head and
+    token) or [T, heads * rows]; ``in_rows``, ``out_rows`` [T, (heads / heads_per_group) * rows]; ``values``
+    [T, heads * cols]; ``bonus`` [heads, rows]; ``value_scale`` [T, heads]; ``skip`` [heads].  Returns y, float32
+    [T, heads * cols]."""
+    tokens = values.shape[0]
+    groups_of_heads = heads // heads_per_group
+    if heads % heads_per_group:
+        raise ValueError(f"{heads} heads in groups of {heads_per_group}")
+    per_row = decay.dim() == 2 and decay.shape[1] == heads * rows and rows > 1
+    for name, t, width in (("decay", decay, heads * rows if per_row else heads), ("in_rows", in_rows, groups_of_heads * rows),
+                           ("out_rows", out_rows, groups_of_heads * rows), ("values", values, heads * cols)):
+        if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1 and tuple(t.shape) == (tokens, width)):
+            raise ValueError(f"{name} must be a float32 GPU view [{tokens}, {width}] with unit inner stride, is {tuple(t.shape)} {t.dtype}")
+    _gpu("state", state, torch.float32, 4)
+    if tuple(state.shape[1:]) != (heads, rows, cols):
+        raise ValueError(f"state {tuple(state.shape)} does not hold {heads} memories of {rows} x {cols}")
+    if bonus is not None:
+        _gpu("bonus", bonus, torch.float32, 2)
+        if tuple(bonus.shape) != (heads, rows) or not read_first:
+            raise ValueError("the bonus is [heads, rows] and comes with a read-out in front of the update")
+    ld_scale = 0
+    if value_scale is not None:
+        if not (value_scale.is_cuda and value_scale.dtype == torch.float32 and tuple(value_scale.shape) == (tokens, heads)
+                and value_scale.stride(1) == 1):
+            raise ValueError(f"value_scale must be float32 [{tokens}, {heads}]")
+        ld_scale = value_scale.stride(0)
+    if skip is not None:
+        _gpu("skip", skip, torch.float32, 1)
+        if skip.shape[0] != heads:
+            raise ValueError(f"skip must be [{heads}]")
+    for name, meta, least in (("seq_slot", seq_slot, sequences), ("q_start_loc", q_start_loc, sequences + 1)):
+        _gpu(name, meta, torch.int32, 1)
+        if meta.shape[0] < least:
+            raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
+    per_thread, row_groups, slice_cols, chunk = plan_memory_walk(rows, cols, per_row, bonus is not None, sequences * heads)
+    y = torch.empty((tokens, heads * cols), dtype=torch.float32, device=values.device)
+    ld = lambda t: t.stride(0) if tokens > 1 else max(t.stride(0), t.shape[1])
+    _run("cie_memory_walk", load_library().cie_memory_walk(
+        _stream(), _ptr(decay), ld(decay), _i(rows if per_row else 1), _i(1 if per_row else 0), _ptr(in_rows), ld(in_rows),
+        _ptr(out_rows), ld(out_rows), _i(heads_per_group), _ptr(bonus), _ptr(values), ld(values), _ptr(value_scale),
+        ld_scale, _ptr(skip), _ptr(state), _ptr(seq_slot), _ptr(q_start_loc), _ptr(y), _i(sequences), _i(heads), _i(rows),
+        _i(cols), _i(per_thread), _i(row_groups), _i(slice_cols), _i(chunk), _i(1 if read_first else 0)))
+    return y
+
+
+def space_steps(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Step sizes and decays of a state-space layer: ``dt = softplus(raw + bias)`` and ``exp(-exp(a_log) * dt)`` per
+    token and head, both float32 [T, heads].  ``raw`` [T, heads] (a view with unit inner stride); bias, a_log float32."""
+    if not (raw.is_cuda and raw.dim() == 2 and raw.stride(1) == 1 and raw.dtype in _CODES):
+        raise ValueError("raw must be a float32 or bfloat16 GPU matrix with unit inner stride")
+    tokens, heads = raw.shape
+    for name, t in (("bias", bias), ("a_log", a_log)):
+        _gpu(name, t, torch.float32, 1)
+        if t.shape[0] != heads:
+            raise ValueError(f"{name} must be [{heads}]")
+    steps = torch.empty((tokens, heads), dtype=torch.float32, device=raw.device)
+    decay = torch.empty((tokens, heads), dtype=torch.float32, device=raw.device)
+    ld = raw.stride(0) if tokens > 1 else max(raw.stride(0), heads)
+    _run("cie_space_steps", load_library().cie_space_steps(_stream(), _i(_code(raw.dtype)), _ptr(raw), ld, _ptr(bias),
+                                                           _ptr(a_log), _ptr(steps), _ptr(decay), _i(tokens), _i(heads)))
+    return steps, decay
+
+
+def shift_mix(h: torch.Tensor, before: torch.Tensor, mu: torch.Tensor, seq_of_token: torch.Tensor,
+              seq_slot: torch.Tensor, q_start_loc: torch.Tensor) -> torch.Tensor:
+    """``mixes[s, t] = h[t] + (h[t - 1] - h[t]) * mu[s]`` within each sequence, [n_mix, T, W] in h's type; the row in
+    front of a step's first token comes from ``before`` (float32 [slots, W]; zeros for a new sequence), which
+    ``time_decay`` moves on.  ``mu`` float32 [n_mix, W]."""
+    if not (h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _CODES):
+        raise ValueError("h must be a float32 or bfloat16 GPU matrix with unit inner stride")
+    tokens, width = h.shape
+    _gpu("before", before, torch.float32, 2)
+    _gpu("mu", mu, torch.float32, 2)
+    if before.shape[1] != width or mu.shape[1] != width:
+        raise ValueError(f"before {tuple(before.shape)} / mu {tuple(mu.shape)} do not fit rows of {width}")
+    for name, meta in (("seq_of_token", seq_of_token), ("seq_slot", seq_slot), ("q_start_loc", q_start_loc)):
+        _gpu(name, meta, torch.int32, 1)
+    if seq_of_token.shape[0] < tokens:
+        raise ValueError("one sequence index per token")
+    mixes = torch.empty((mu.shape[0], tokens, width), dtype=h.dtype, device=h.device)
+    ldh = h.stride(0) if tokens > 1 else max(h.stride(0), width)
+    _run("cie_shift_mix", load_library().cie_shift_mix(_stream(), _i(_code(h.dtype)), _ptr(h), ldh, _ptr(before), _ptr(mu),
+                                                       _ptr(seq_of_token), _ptr(seq_slot), _ptr(q_start_loc), _ptr(mixes),
+                                                       _i(tokens), _i(width), _i(mu.shape[0])))
+    return mixes
+
+
+def time_decay(low: torch.Tensor, w2: torch.Tensor, w0: torch.Tensor, h: torch.Tensor, before: torch.Tensor,
+               seq_of_token: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor) -> torch.Tensor:
+    """``exp(-exp(w2 tanh(low) + w0))``, float32 [T, C]: ``low`` float32 [T, rank], ``w2`` [C, rank] in h's type,
+    ``w0`` float32 [C].  Also leaves the last row of ``h`` of every sequence of the step in ``before`` (the token-shift
+    state that ``shift_mix`` reads at the next step)."""
+    _gpu("low", low, torch.float32, 2)
+    tokens, rank = low.shape
+    if not (h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _CODES and h.shape[0] == tokens):
+        raise ValueError("h must be a float32 or bfloat16 GPU matrix with unit inner stride, a row per token")
+    _gpu("w2", w2, h.dtype, 2)
+    channels = w2.shape[0]
+    _gpu("w0", w0, torch.float32, 1)
+    _gpu("before", before, torch.float32, 2)
+    if w2.shape[1] != rank or w0.shape[0] != channels or before.shape[1] != h.shape[1]:
+        raise ValueError(f"w2 {tuple(w2.shape)}, w0 {tuple(w0.shape)}, before {tuple(before.shape)} do not fit")
+    for name, meta in (("seq_of_token", seq_of_token), ("seq_slot", seq_slot), ("q_start_loc", q_start_loc)):
+        _gpu(name, meta, torch.int32, 1)
+    decay = torch.empty((tokens, channels), dtype=torch.float32, device=low.device)
+    ldh = h.stride(0) if tokens > 1 else max(h.stride(0), h.shape[1])
+    _run("cie_time_decay", load_library().cie_time_decay(
+        _stream(), _i(_code(h.dtype)), _ptr(low), _ptr(w2), _ptr(w0), _ptr(decay), _i(tokens), _i(channels), _i(rank),
+        _ptr(h), ldh, _ptr(before), _ptr(seq_of_token), _ptr(seq_slot), _ptr(q_start_loc), _i(h.shape[1])))
+    return decay
+
+
+def gated_group_norm(y: torch.Tensor, gate: Optional[torch.Tensor], weight: Optional[torch.Tensor], groups: int,
+                     eps: float, out_dtype: torch.dtype, gate_first: bool) -> torch.Tensor:
+    """The RMS norm of float32 rows ``y`` [T, W] in ``groups`` equal consecutive parts (each over its own root mean
+    square), times ``weight`` (float32 [W]), with ``silu(gate)`` multiplied in front of the norm (``gate_first``) or
+    behind it.  ``gate`` [T, W] in ``out_dtype`` (a view with unit inner stride)."""
+    _gpu("y", y, torch.float32, 2)
+    tokens, width = y.shape
+    if groups < 1 or width % groups or not eps > 0 or width + groups > MAX_NORM_WIDTH:
+        raise ValueError(f"{groups} groups over rows of {width} with eps {eps}")
+    ldg = 0
+    if gate is not None:
+        if not (gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.dtype == out_dtype
+                and tuple(gate.shape) == (tokens, width)):
+            raise ValueError(f"gate must be a [{tokens}, {width}] view of {out_dtype} with unit inner stride")
+        ldg = gate.stride(0) if tokens > 1 else max(gate.stride(0), width)
+    if weight is not None:
+        _gpu("weight", weight, torch.float32, 1)
+        if weight.shape[0] != width:
+            raise ValueError(f"weight must be [{width}]")
+    out = torch.empty((tokens, width), dtype=out_dtype, device=y.device)
+    _run("cie_gated_group_norm", load_library().cie_gated_group_norm(
+        _stream(), _i(_code(out_dtype)), _ptr(y), _ptr(gate), ldg, _ptr(weight), _ptr(out), _i(tokens), _i(width),
+        _i(groups), _f(eps), _i(1 if gate_first else 0)))
+    return out
+
+
+# ---------------------------------------------------------------------------
 def branch_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                    out_dtype: torch.dtype, parts: Optional[torch.Tensor] = None,
-                    want_rows: bool = True) -> Optional[torch.Tensor]:
-    """``residual += y / sqrt(mean(y^2) + eps) * weight`` with ``y = branch + sum_p parts[:, p]``, row by row, in
-    float32 and in place.  ``branch`` [T, H] float32 or ``out_dtype`` (or ``None``), ``parts`` float32 [T, P, H]
-    (or ``None``), ``weight`` float32 [H] as it multiplies.  Returns the new stream rounded to ``out_dtype``
-    (``want_rows``), which is what the next sublayer's products read."""
+                    out_dtype: torch.dtype, parts: Optional[torch.Tensor] = None, want_rows: bool = True,
+                    branch_gate: Optional[torch.Tensor] = None, part_weight: Optional[torch.Tensor] = None,
+                    branch2: Optional[torch.Tensor] = None, scales: tuple[float, float] = (1.0, 1.0),
+                    next_weight: Optional[torch.Tensor] = None):
+    """``residual += y / sqrt(mean(y^2) + eps) * weight`` with ``y = scales[0] * branch * sigmoid(branch_gate) +
+    scales[1] * branch2 + sum_p part_weight[:, p] * parts[:, p]`` (whatever of it is given), row by row, in float32
+    and in place.  ``branch``, ``branch2`` [T, H] float32 or ``out_dtype``; ``branch_gate`` float32 [T] (logits, any
+    stride); ``parts`` float32 [T, P, H]; ``part_weight`` float32 [T, P]; ``weight`` float32 [H] as it multiplies.
+    Returns the new stream rounded to ``out_dtype`` (``want_rows``), which is what a sublayer that reads the stream
+    itself takes; with ``next_weight`` (float32 [H]) a pair of that and the RMS norm of the new stream under that
+    weight, in ``out_dtype``."""
     _gpu("residual", residual, torch.float32, 2)
     tokens, hidden = residual.shape
     _gpu("weight", weight, torch.float32, 1)
     if not (weight.shape[0] == hidden and hidden <= MAX_NORM_WIDTH and eps > 0):
         raise ValueError(f"weight {tuple(weight.shape)}, hidden {hidden}, eps {eps} do not fit the norm kernel")
-    if branch is None and parts is None:
+    if branch is None and parts is None and branch2 is None:
         raise ValueError("nothing to add")
-    if branch is not None:
-        _gpu("branch", branch, dims=2)
-        if not (branch.shape == residual.shape and branch.dtype in (torch.float32, out_dtype)):
-            raise ValueError(f"branch {tuple(branch.shape)} {branch.dtype} does not fit {tuple(residual.shape)} {out_dtype}")
+    kinds = set()
+    for name, t in (("branch", branch), ("branch2", branch2)):
+        if t is not None:
+            _gpu(name, t, dims=2)
+            if not (t.shape == residual.shape and t.dtype in (torch.float32, out_dtype)):
+                raise ValueError(f"{name} {tuple(t.shape)} {t.dtype} does not fit {tuple(residual.shape)} {out_dtype}")
+            kinds.add(t.dtype)
+    if len(kinds) > 1:
+        raise ValueError("the two branches must be of one type")
+    gate_stride = 1
+    if branch_gate is not None:
+        if not (branch_gate.is_cuda and branch_gate.dtype == torch.float32 and branch_gate.dim() == 1):
+            raise ValueError("branch_gate must be a float32 GPU vector")
+        if branch is None or branch_gate.shape[0] != tokens:
+            raise ValueError("a gate comes with a branch, one logit per row")
+        gate_stride = max(branch_gate.stride(0), 1)
     n_parts = 0
     if parts is not None:
         _gpu("parts", parts, torch.float32, 3)
         if not (parts.shape[0] == tokens and parts.shape[2] == hidden):
             raise ValueError(f"parts {tuple(parts.shape)} do not fit {tuple(residual.shape)}")
         n_parts = parts.shape[1]
+    if part_weight is not None:
+        _gpu("part_weight", part_weight, torch.float32)
+        if parts is None or part_weight.numel() != tokens * n_parts:
+            raise ValueError("part weights come with parts, one per part and row")
+    normed = None
+    if next_weight is not None:
+        _gpu("next_weight", next_weight, torch.float32, 1)
+        if next_weight.shape[0] != hidden:
+            raise ValueError(f"next_weight must be [{hidden}]")
+        normed = torch.empty((tokens, hidden), dtype=out_dtype, device=residual.device)
     rows = torch.empty((tokens, hidden), dtype=out_dtype, device=residual.device) if want_rows else None
+    kind = kinds.pop() if kinds else torch.float32
     _run("cie_branch_norm_add", load_library().cie_branch_norm_add(
-        _stream(), _i(_code(branch.dtype if branch is not None else torch.float32)), _i(_code(out_dtype)),
-        _ptr(residual), _ptr(branch), _ptr(parts), _i(n_parts), _ptr(weight), _ptr(rows), _i(tokens), _i(hidden), _f(eps)))
-    return rows
+        _stream(), _i(_code(kind)), _i(_code(out_dtype)), _ptr(residual), _ptr(branch), _ptr(branch_gate),
+        _i(gate_stride), _ptr(branch2), _f(scales[0]), _f(scales[1]), _ptr(parts), _ptr(part_weight), _i(n_parts),
+        _ptr(weight), _ptr(rows), _i(tokens), _i(hidden), _f(eps), _ptr(next_weight), _ptr(normed)))
+    return rows if next_weight is None else (rows, normed)
 
 
 def group_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weight: torch.Tensor, groups: int, eps: float,
@@ -1191,16 +1419,18 @@ def group_norm_add(residual: torch.Tensor, branch: Optional[torch.Tensor], weigh
     return out
 
 
-def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, offset: float) -> torch.Tensor:
-    """``g * sigmoid(alpha * g) * (u + offset)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)`` for
-    gate_up [T, 2I] (gate half first)."""
+def clamped_glu(gate_up: torch.Tensor, limit: float, alpha: float, offset: float, cubic: float = 0.0) -> torch.Tensor:
+    """``g * sigmoid(alpha * (g + cubic * g^3)) * (u + offset)`` with ``g = min(gate, limit)``,
+    ``u = clamp(up, -limit, limit)`` for gate_up [T, 2I] (gate half first).  ``cubic = 0`` is the plain sigmoid
+    gate; ``alpha = 2 sqrt(2 / pi)`` with ``cubic = 0.044715`` is the tanh form of gelu."""
     _gpu("gate_up", gate_up, dims=2)
     tokens, twice = gate_up.shape
     if twice % 2 or not limit > 0:
         raise ValueError(f"gate_up rows must be even and the limit positive, got {twice}, {limit}")
     out = torch.empty((tokens, twice // 2), dtype=gate_up.dtype, device=gate_up.device)
     _run("cie_clamped_glu", load_library().cie_clamped_glu(_stream(), _i(_code(gate_up.dtype)), _ptr(gate_up), _ptr(out),
-                                                           _i(tokens), _i(twice // 2), _f(limit), _f(alpha), _f(offset)))
+                                                           _i(tokens), _i(twice // 2), _f(limit), _f(alpha), _f(offset),
+                                                           _f(cubic)))
     return out
 
 
@@ -1214,7 +1444,7 @@ def soft_cap_(x: torch.Tensor, cap: float) -> torch.Tensor:
 
 
 # ---------------------------------------------------------------------------
-NORM_MODES = {None: 0, "unit": 1, "weight": 2}
+NORM_MODES = {None: 0, "unit": 1, "weight": 2, "whole": 3}
 SCORED_MFMA_DIMS = ((64, 64), (128, 128), (64, 128), (128, 64))  # (key, value) head sizes of the matrix-core form
 
 
@@ -1237,7 +1467,8 @@ def heads_prepare(proj: torch.Tensor, offsets: tuple[int, int, int], q_heads: in
     """From projected rows ``proj`` [T, >= ...] (queries at column ``offsets[0]``, keys at ``offsets[1]``, values at
     ``offsets[2]``, heads of ``dim`` / ``dim`` / ``vdim`` numbers) to queries ``[T, q_heads * kernel_dim]`` and the
     token's cache entries: per-head RMS norm of queries and keys (``norm``: ``None``, ``"unit"`` or ``"weight"`` with
-    float32 weights [dim]), the queries times ``1 + coef * ln(floor((p + 1) / every) + 1)`` (``temperature = (coef,
+    float32 weights [dim]; or ``"whole"``: over all query heads together and over all key heads together, weights
+    [q_heads * dim] and [kv_heads * dim]), the queries times ``1 + coef * ln(floor((p + 1) / every) + 1)`` (``temperature = (coef,
     every)``), heads zero-padded up to the kernels' sizes.  ``rotary = (cos, sin, rot, neighbours)``: after the norm
     the first ``rot`` numbers of every query and key head turn by the token's position, in pairs of neighbours
     ``(2i, 2i + 1)`` or of the halves ``(i, i + rot / 2)``; cos and sin are float32 ``[positions, rot / 2]`` and must
@@ -1246,18 +1477,24 @@ def heads_prepare(proj: torch.Tensor, offsets: tuple[int, int, int], q_heads: in
         raise ValueError("proj must be 2-d on the GPU with unit inner stride")
     dtype = proj.dtype
     q_off, k_off, v_off = offsets
-    need = max(q_off + q_heads * dim, k_off + kv_heads * dim, v_off + kv_heads * vdim)
+    need = q_off + q_heads * dim
+    if write_kv:
+        need = max(need, k_off + kv_heads * dim, v_off + kv_heads * vdim)
     if not (proj.shape[0] >= tokens and proj.shape[1] >= need and min(offsets) >= 0):
         raise ValueError(f"proj {tuple(proj.shape)} too small for {tokens} tokens of {need} numbers")
     if norm not in NORM_MODES:
         raise ValueError(f"norm must be one of {list(NORM_MODES)}, got {norm!r}")
-    if norm == "weight":
-        for name, w in (("q_weight", q_weight), ("k_weight", k_weight)):
+    if norm in ("weight", "whole"):
+        # ("whole": one root mean square over all query heads of a token and one over all its key heads, a weight per
+        # number of the projection; a call that writes no keys needs no key weight)
+        for name, w, heads in (("q_weight", q_weight, q_heads), ("k_weight", k_weight, kv_heads)):
+            if w is None and name == "k_weight" and not write_kv:
+                continue
             if w is None:
                 raise ValueError(f"{name} is missing")
             _gpu(name, w, torch.float32, 1)
-            if w.shape[0] != dim:
-                raise ValueError(f"{name} must be [{dim}], is {tuple(w.shape)}")
+            if w.shape[0] != (dim if norm == "weight" else heads * dim):
+                raise ValueError(f"{name} {tuple(w.shape)} does not fit heads of {dim} under the {norm!r} norm")
     if kernel_dim < dim or kernel_vdim < vdim:
         raise ValueError("the kernels' head sizes must hold the projection's")
     page_size = _check_kv_pools(k_pool, v_pool, dtype, kv_heads, kernel_dim, kernel_vdim)
@@ -1290,9 +1527,11 @@ def heads_prepare(proj: torch.Tensor, offsets: tuple[int, int, int], q_heads: in
     return q_out
 
 
-def _check_score_shape(q_heads: int, slopes, sinks, softcap, window=None, chunk=None) -> None:
+def _check_score_shape(q_heads: int, slopes, sinks, softcap, window=None, chunk=None, keep_first=0) -> None:
     if chunk is not None and (chunk < 1 or window):
         raise ValueError(f"chunks hold at least one token and stand in a window's place, got chunk {chunk}, window {window}")
+    if keep_first < 0 or (keep_first and not window):
+        raise ValueError(f"kept first keys ({keep_first}) are a count and come with a window")
     for name, t in (("slopes", slopes), ("sinks", sinks)):
         if t is not None:
             _gpu(name, t, torch.float32, 1)
@@ -1316,9 +1555,10 @@ def scored_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torc
                              q_heads: int, kv_heads: int, dim: int, vdim: int, window: Optional[int], scale: float,
                              softcap: Optional[float] = None, slopes: Optional[torch.Tensor] = None,
                              sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                             chunk: Optional[int] = None) -> torch.Tensor:
+                             chunk: Optional[int] = None, keep_first: int = 0) -> torch.Tensor:
     """Attention of each token over its request's cached keys with shaped scores (see ``csrc/attention_scored.hip``;
-    ``chunk``: a token sees the keys of its own chunk of that many positions, counted from position 0, up to itself):
+    ``chunk``: a token sees the keys of its own chunk of that many positions, counted from position 0, up to itself;
+    ``keep_first``: beside its window a token sees the first that many keys of its sequence):
     ``q`` [T, q_heads * dim]; returns [T, q_heads * vdim].  ``gate`` [T, >= q_heads] (a view is fine): head h's output
     is multiplied by ``sigmoid(gate[t, h])``.  float32 or bfloat16."""
     _gpu("q", q, dims=2)
@@ -1332,14 +1572,14 @@ def scored_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torc
         if not (meta.shape[0] >= tokens):
             raise ValueError(f"{name} has {meta.shape[0]} entries for {tokens} tokens")
     _gpu("seq_slot", seq_slot, torch.int32, 1)
-    _check_score_shape(q_heads, slopes, sinks, softcap, window, chunk)
+    _check_score_shape(q_heads, slopes, sinks, softcap, window, chunk, keep_first)
     gate_stride = _check_gate(gate, tokens, q_heads, q.dtype)
     out = torch.empty((tokens, q_heads * vdim), dtype=q.dtype, device=q.device)
     _run("cie_scored_attention_generic", load_library().cie_scored_attention_generic(
         _stream(), _i(_code(q.dtype)), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), _i(block_table.shape[1]),
         _ptr(positions), _ptr(seq_of_token), _ptr(seq_slot), _ptr(gate), _i(gate_stride), _ptr(out), _i(tokens),
         _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(page_size), _i(window or 0), _f(scale), _f(softcap or 0.0),
-        _ptr(slopes), _ptr(sinks), _i(chunk or 0)))
+        _ptr(slopes), _ptr(sinks), _i(chunk or 0), _i(keep_first)))
     return out
 
 
@@ -1350,7 +1590,8 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
                           tokens_per_tile: int, row_tiles: int, window: Optional[int], scale: float,
                           softcap: Optional[float] = None, slopes: Optional[torch.Tensor] = None,
                           sinks: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
-                          n_splits: int = 1, keys_per_split: int = 0, chunk: Optional[int] = None) -> torch.Tensor:
+                          n_splits: int = 1, keys_per_split: int = 0, chunk: Optional[int] = None,
+                          keep_first: int = 0) -> torch.Tensor:
     """The same on the matrix cores (bfloat16, (dim, vdim) in ``SCORED_MFMA_DIMS``, pages of a power of two >= 4):
     tiles of ``tokens_per_tile`` consecutive tokens of one sequence (``tile_seq``, ``tile_q0`` int32 [n_tiles]; both
     ``None``: tile i is sequence i's first), whose rows times the heads per key head fill ``row_tiles`` tiles of 16.
@@ -1381,7 +1622,7 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
             raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
     if tile_seq is None and n_tiles > sequences:
         raise ValueError(f"{n_tiles} tiles for {sequences} sequences")
-    _check_score_shape(q_heads, slopes, sinks, softcap, window, chunk)
+    _check_score_shape(q_heads, slopes, sinks, softcap, window, chunk, keep_first)
     gate_stride = _check_gate(gate, tokens, q_heads, q.dtype)
     out = torch.empty((tokens, q_heads * vdim), dtype=q.dtype, device=q.device)
     part_o = part_ml = None
@@ -1398,7 +1639,7 @@ def scored_attention_mfma(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.T
         _ptr(tile_q0), _i(n_tiles), _ptr(seq_slot), _ptr(seq_start), _ptr(seq_q_len), _ptr(q_start_loc), _ptr(gate),
         _i(gate_stride), _ptr(out), _i(q_heads), _i(kv_heads), _i(dim), _i(vdim), _i(page_size), _i(tokens_per_tile),
         _i(row_tiles), _i(window or 0), _f(scale), _f(softcap or 0.0), _ptr(slopes), _ptr(sinks), _i(n_splits),
-        _i(keys_per_split), _ptr(part_o), _ptr(part_ml), _i(chunk or 0)))
+        _i(keys_per_split), _ptr(part_o), _ptr(part_ml), _i(chunk or 0), _i(keep_first)))
     return out
 
 

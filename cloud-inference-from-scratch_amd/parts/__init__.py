@@ -1,5 +1,5 @@
-from . import (attention, block, feed_forward, latent_attention, norm, position, recurrent,  # noqa: F401
-               routed_experts, scored_attention)  # (fill the registries)
+from . import (attention, block, feed_forward, latent_attention, norm, parallel_mixers, position,  # noqa: F401
+               recurrent, routed_experts, scored_attention)  # (fill the registries)
 from .base import (
     BLOCKS,
     FEED_FORWARDS,

@@ -11,6 +11,9 @@ cheaper form or rides along with the product behind it (``parts/linear.py``).
 ``BranchNormBlock``: the sublayers read the stream itself and their outputs are normed before they are added:
 ``h += norm1(mixer(h)); h += norm2(feed_forward(h))``.
 
+``SandwichNormBlock``: a norm in front of every sublayer and one on its output, which is then scaled per channel:
+``h += s1 * norm1_out(mixer(norm1(h))); h += s2 * norm2_out(feed_forward(norm2(h)))``.
+
 ``ParallelDepthBlock``: both branches read the same stream, and the next layer reads a weighted average of what
 the embedding and all layers so far left (below).
 """
@@ -26,7 +29,7 @@ from ..config.specs import LayerSpec
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import build_part, register_part
-from .linear import Added, RawRows, RowSumsq, StreamRows
+from .linear import Added, RawRows, RowSumsq, StreamRows, WeightedPair
 
 
 class PreNormBlock:
@@ -111,6 +114,8 @@ def normalise(norm, residual: torch.Tensor, pending, dtype: torch.dtype, rows=No
     other an already added branch becomes ``None``."""
     if not getattr(norm, "takes_row_sumsq", False) and isinstance(pending, (RowSumsq, Added)):
         pending = None
+    if isinstance(pending, WeightedPair):
+        pending = pending.combined()
     if rows is not None:
         return norm.forward(residual, pending, dtype, rows=rows)
     return norm.forward(residual, pending, dtype)
@@ -273,3 +278,86 @@ class ParallelDepthBlock:
 
 
 register_part("block", "parallel_depth_average", ParallelDepthBlock)
+
+
+class SandwichNormBlock(PreNormBlock):
+    """``h += s1 * norm1_out(mixer(norm1(h)))``, then ``h += s2 * norm2_out(feed_forward(norm2(h)))``: norms on both
+    sides of a sublayer, and a learned scale per channel (``s1``, ``s2``: the checkpoint tensors ``<layer>ls1`` and
+    ``<layer>ls2``, or whatever the spec's ``names`` call ``scale1`` and ``scale2``) on what joins the stream.  The
+    scale is folded into the output norm's weight once, in float32.  One kernel norms a sublayer's output, adds it
+    and makes the norm that the next sublayer reads (the next layer's first norm too, where that layer is of this
+    kind), so the stream is read and written once per sublayer.  The output norms are of a kind with ``add_normed``
+    (``rms_norm_groups`` with one group).  A layer without feed-forward has neither second norm nor ``s2``."""
+
+    def __init__(self, spec: LayerSpec) -> None:
+        super().__init__(spec)
+        if spec.norm1_out is None or (self.has_feed_forward and spec.norm2_out is None):
+            raise ValueError("this arrangement needs a norm for every sublayer's output (norm1_out, norm2_out)")
+        self.norm1_out = build_part("norm", spec.norm1_out)
+        self.norm2_out = build_part("norm", spec.norm2_out) if self.has_feed_forward else None
+        self.layer_scale = bool(spec.option("layer_scale", True))
+        for norm in (self.norm1_out, self.norm2_out):
+            if norm is not None and not hasattr(norm, "add_normed"):
+                raise ValueError("this arrangement takes output norms that can add a normed branch")
+        self.next_block: Any = None
+
+    def link_next(self, block: Any) -> None:
+        """The block that runs after this one (``None``: the last); its first norm rides in this block's last kernel."""
+        self.next_block = block if isinstance(block, SandwichNormBlock) else None
+
+    def _parts(self):
+        parts = [("norm1", self.norm1), ("mixer", self.mixer), ("norm1_out", self.norm1_out)]
+        if self.has_feed_forward:
+            parts += [("norm2", self.norm2), ("feed_forward", self.feed_forward), ("norm2_out", self.norm2_out)]
+        return parts
+
+    def _scales(self):
+        if not self.layer_scale:
+            return ()
+        return ("scale1", "scale2") if self.has_feed_forward else ("scale1",)
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        out = super().expected_tensors(prefix)
+        width = self.norm1.size
+        for role in self._scales():
+            out[prefix + self.spec.name_of(role)] = TensorSpec((width,), init="norm", keeps_float32=True)
+        if not self.has_feed_forward:
+            extra = dict(build_part("norm", self.spec.norm2_out).expected_tensors(f"{prefix}{self.spec.name_of('norm2_out')}.")
+                         if self.spec.norm2_out is not None else {})
+            if self.layer_scale:
+                extra[prefix + self.spec.name_of("scale2")] = TensorSpec((width,), init="norm", keeps_float32=True)
+            for name, spec in extra.items():
+                out[name] = replace(spec, optional=True)
+        return out
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        # the scale per channel and the output norm's weight multiply one after the other: their float32 product, once
+        self.out_weight1 = self.norm1_out.weight_f32
+        self.out_weight2 = self.norm2_out.weight_f32 if self.has_feed_forward else None
+        if self.layer_scale:
+            self.out_weight1 = (self.out_weight1 * tensors[prefix + self.spec.name_of("scale1")].float()).contiguous()
+            if self.has_feed_forward:
+                self.out_weight2 = (self.out_weight2 * tensors[prefix + self.spec.name_of("scale2")].float()).contiguous()
+
+    def forward(self, residual: torch.Tensor, pending, batch, view, writes: bool = True):
+        if isinstance(pending, NormedRows) and pending.owner is self:
+            x = pending.first
+        else:
+            x = normalise(self.norm1, residual, pending, self.dtype)
+        mixed = self.mixer.forward(x, batch, view, writes)
+        follower = self.next_block
+        after = follower.norm1.weight_f32 if follower is not None else None
+        if self.has_feed_forward:
+            _, x = self.norm1_out.add_normed(residual, mixed, self.dtype, weight=self.out_weight1,
+                                             then=self.norm2.weight_f32)
+            fed = self.feed_forward.forward(x)
+            last = self.norm2_out.add_normed(residual, fed, self.dtype, weight=self.out_weight2, then=after)
+        else:
+            last = self.norm1_out.add_normed(residual, mixed, self.dtype, weight=self.out_weight1, then=after)
+        if follower is None:
+            return residual, None
+        return residual, NormedRows(last[1], None, follower)
+
+
+register_part("block", "sandwich_norm", SandwichNormBlock)

@@ -53,17 +53,19 @@ class ClampedGatedMLP(Part):
     """A dense gated feed-forward whose unit bounds its inputs: ``g = min(W_gate x, limit)``,
     ``u = clamp(W_up x, -limit, limit)``, ``y = W_down (g * sigmoid(alpha g) * (u + offset))``.  ``limit``, ``alpha``
     and ``offset`` are parameters (``limit=None``: unbounded; ``alpha=1, offset=0`` is ``silu(g) * u``); the unit is
-    computed in float32 from the product's rows."""
+    computed in float32 from the product's rows.  ``cubic`` puts ``g + cubic * g^3`` inside the sigmoid:
+    ``alpha = 2 sqrt(2 / pi)`` with ``cubic = 0.044715`` is the tanh form of gelu on the gate (``GELU_TANH``)."""
 
     graph_safe = True
+    GELU_TANH = dict(alpha=2.0 * (2.0 / 3.141592653589793) ** 0.5, cubic=0.044715, offset=0.0)
 
     def __init__(self, hidden_size: int, intermediate_size: int, limit: Optional[float] = None, alpha: float = 1.0,
-                 offset: float = 0.0, names: tuple[str, str, str] = ("gate", "up", "down")) -> None:
+                 offset: float = 0.0, names: tuple[str, str, str] = ("gate", "up", "down"), cubic: float = 0.0) -> None:
         if min(hidden_size, intermediate_size) < 1 or (limit is not None and not limit > 0):
             raise ValueError("sizes and the limit must be positive")
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
         self.limit = float("inf") if limit is None else float(limit)
-        self.alpha, self.offset = float(alpha), float(offset)
+        self.alpha, self.offset, self.cubic = float(alpha), float(offset), float(cubic)
         self.names = tuple(names)
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
@@ -84,7 +86,7 @@ class ClampedGatedMLP(Part):
         self.forward(torch.zeros((rows, self.hidden_size), dtype=self.w_down.dtype, device=self.w_down.device))
 
     def forward(self, x, residual: Optional[torch.Tensor] = None):
-        hidden = ops.clamped_glu(linear(x, self.w_gate_up), self.limit, self.alpha, self.offset)
+        hidden = ops.clamped_glu(linear(x, self.w_gate_up), self.limit, self.alpha, self.offset, self.cubic)
         return linear(hidden, self.w_down)
 
 

@@ -157,6 +157,21 @@ class SummedBranch:
 
 
 @dataclass
+class WeightedPair:
+    """A branch output that is still a weighted sum of two: ``scales[0] * first + scales[1] * second`` (two mixers
+    that ran side by side).  A block whose adding kernel takes two branches hands them over as they are; any other
+    asks for :meth:`combined`."""
+
+    first: torch.Tensor
+    second: torch.Tensor
+    scales: tuple[float, float] = (1.0, 1.0)
+
+    def combined(self) -> torch.Tensor:
+        total = self.first.float() * self.scales[0] + self.second.float() * self.scales[1]
+        return total.to(self.first.dtype)
+
+
+@dataclass
 class RawRows:
     """Stands where an RMSNorm's output would, before anything was computed: the rows are the norm ``norm``
     of the float32 stream ``residual``.  Only a mixer that says ``takes_raw_rows`` is shown it (the attention

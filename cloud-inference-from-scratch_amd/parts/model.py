@@ -77,10 +77,21 @@ class DecoderModel:
                 needs[call.cache] = need
                 seen.add(call.cache)
         for call in self.spec.order:
-            if not call.writes and self.blocks[call.layer].cache_need() != needs[call.cache]:
+            if call.writes:
+                continue
+            need = self.blocks[call.layer].cache_need()
+            if need == needs[call.cache]:
+                continue
+            # a reader with a mask of its own: the unit keeps what either of them still sees
+            join = getattr(needs[call.cache], "joined", None)
+            try:
+                if join is None or type(need) is not type(needs[call.cache]):
+                    raise ValueError("not a paged cache on both sides")
+                needs[call.cache] = join(need)
+            except ValueError as error:
                 raise ValueError(
-                    f"layer {call.layer} reads cache unit {call.cache} whose shape it does not share"
-                )
+                    f"layer {call.layer} reads cache unit {call.cache} whose shape it does not share ({error})"
+                ) from error
         return needs
 
     @property

@@ -15,7 +15,7 @@ import torch
 from ..kernels import ops
 from ..weights.tensors import TensorSpec
 from .base import Part, register_part
-from .linear import Added, RowSumsq, ScaledRows, SummedBranch
+from .linear import Added, RowSumsq, ScaledRows, SummedBranch, WeightedPair
 
 
 class RMSNorm(Part):
@@ -152,6 +152,28 @@ class GroupedRMSNorm(Part):
         return ops.group_norm_add(residual, branch, self.weight, self.groups, self.eps, out_dtype, rows=rows,
                                   plus=plus, **extra)
 
+
+def _add_normed(self, residual: torch.Tensor, branch, out_dtype: torch.dtype, want_rows: bool = False,
+                weight: Optional[torch.Tensor] = None, then: Optional[torch.Tensor] = None):
+    """``residual += norm(branch) * weight`` in float32 and in place, for a norm of one group.  ``branch``: a
+    tensor, a ``SummedBranch`` (rows still to be summed, with their weights and the gate on its main tensor) or a
+    ``WeightedPair``.  ``weight`` (float32 [H]) stands in for the norm's own where the caller has folded a scale per
+    channel into it.  ``then`` (float32 [H]): the RMS norm of the new stream under that weight comes back too.
+    Returns what ``ops.branch_norm_add`` returns."""
+    if self.groups != 1:
+        raise ValueError("a norm on a sublayer's output takes its statistics over the whole row")
+    extra = {}
+    if isinstance(branch, SummedBranch):
+        extra = dict(parts=branch.parts, part_weight=branch.weights, branch_gate=branch.main_gate)
+        branch = branch.main
+    elif isinstance(branch, WeightedPair):
+        extra = dict(branch2=branch.second, scales=branch.scales)
+        branch = branch.first
+    return ops.branch_norm_add(residual, branch, self.weight if weight is None else weight, self.eps, out_dtype,
+                               want_rows=want_rows, next_weight=then, **extra)
+
+
+GroupedRMSNorm.add_normed = _add_normed
 
 register_part("norm", "rms_norm", RMSNorm)
 register_part("norm", "rms_norm_groups", GroupedRMSNorm)

@@ -16,7 +16,8 @@ pairs for contexts beyond the ``original`` length the frequencies were made for:
 ``lo = max(floor(turn(fast)), 0)``, ``hi = min(ceil(turn(slow)), R - 1)`` and
 ``ramp_j = clamp((j - lo) / max(hi - lo, 0.001), 0, 1)``, pair j turns at
 ``inv_freq_j * (1 - ramp_j) + inv_freq_j / factor * ramp_j``, and cos and sin are both multiplied by
-``0.1 ln(factor) + 1``.  ``max_position=None`` is a model without a longest position: the tables then grow as
+``0.1 ln(factor) + 1``.  ``scaling=(factor,)`` alone divides every frequency by the factor and leaves cos and sin as
+they are.  ``max_position=None`` is a model without a longest position: the tables then grow as
 positions are asked for (``tables(device, upto)``), in powers of two.
 """
 
@@ -48,8 +49,8 @@ class RotaryHalf(Part):
             raise ValueError("rotary theta and max_position must be positive")
         if scaling is not None:
             scaling = tuple(float(v) for v in scaling)
-            if len(scaling) != 4 or not all(v > 0 for v in scaling) or theta == 1.0:
-                raise ValueError(f"scaling is (factor, original, fast, slow), all positive, got {scaling}")
+            if len(scaling) not in (1, 4) or not all(v > 0 for v in scaling) or (len(scaling) == 4 and theta == 1.0):
+                raise ValueError(f"scaling is (factor,) or (factor, original, fast, slow), all positive, got {scaling}")
         self.head_dim = head_dim
         self.rotary_dim = rotary_dim
         self.theta = float(theta)
@@ -64,6 +65,8 @@ class RotaryHalf(Part):
         )
         if self.scaling is None:
             return inv_freq, 1.0
+        if len(self.scaling) == 1:
+            return inv_freq / self.scaling[0], 1.0
         factor, original, fast, slow = self.scaling
         turn = lambda t: self.rotary_dim * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(self.theta))
         lo = max(math.floor(turn(fast)), 0)

@@ -15,7 +15,18 @@ norm with a weight over all heads' read-outs together and a ``sigmoid`` gate.
 ``S_t = a S_(t-1) + sqrt(1 - a^2) i u_t``; the output is ``W_o (S_t y_t)``.  Its state is ``S`` [width] and the
 convolution's last ``taps - 1`` inputs, both float32.
 
-Both read their sequences' slots and lengths from the step's device tensors (``csrc/recurrent.hip``), run a step's
+``StateSpace``: a state-space layer with one decay per head and token (the duality form): one product makes
+``z | x | B | C | dt``; ``x, B, C`` pass a causal convolution and ``silu``; ``dt = softplus(dt + bias)``; per head
+``S_t = exp(-exp(A_log) dt) S_(t-1) + dt B_t x_t^T`` and ``y_t = S_t^T C_t + D x_t``; ``y silu(z)`` is normed in
+groups, weighted and projected.  Its state is ``S`` [heads, state, vdim] and the convolution's last inputs.
+
+``TimeMixing``: a memory with a decay per key channel that the token itself sets.  Every projection reads its own
+mix of the token's input and the one before it; ``o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t``, then
+``S_t = diag(w_t) S_(t-1) + k_t v_t^T`` with ``w = exp(-exp(W_2 tanh(W_1 mix) + w_0))``; each head's ``o`` is divided by
+its root mean square, weighted, gated by ``silu`` and projected.  Its state is ``S`` [heads, dim, dim] and the input
+of the token before.
+
+These two run the same walk (``ops.memory_walk``).  All of them read their sequences' slots and lengths from the step's device tensors (``csrc/recurrent.hip``), run a step's
 tokens in order from the state the earlier steps left and write it back, so a prompt may be cut anywhere.
 """
 
@@ -225,6 +236,164 @@ class GatedLinearRecurrence(Part):
         return linear(out, self.w_o)
 
 
+class StateSpace(Part):
+    """``W_in x`` is laid out ``[z: inner | x: inner | B: groups * state | C: groups * state | dt: heads]`` with
+    ``inner = heads * vdim``; head h uses the B and C of group ``h // (heads / groups)``.  Tensors: ``in``, ``conv``
+    [inner + 2 groups state, taps] with ``conv.b`` (the last tap is the token's own input), ``dt_bias``, ``A_log``,
+    ``D`` [heads], ``norm`` [inner], ``o``.  The gate ``silu(z)`` comes before the norm, which runs over
+    ``norm_groups`` equal parts of the row.  Products and the convolution with its activation run in the engine's
+    type; step sizes, decays, the memory, the read-out and the norm are float32."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, value_dim: int, state: int, groups: int, taps: int,
+                 norm_groups: int, eps: float) -> None:
+        for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("value_dim", value_dim),
+                            ("state", state), ("groups", groups), ("taps", taps), ("norm_groups", norm_groups)):
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be a positive integer, got {value!r}")
+        if num_heads % groups or (num_heads * value_dim) % norm_groups:
+            raise ValueError(f"{num_heads} heads of {value_dim} in {groups} groups, normed in {norm_groups} parts: no equal parts")
+        if taps > ops.MAX_CONV_TAPS or not eps > 0:
+            raise ValueError(f"up to {ops.MAX_CONV_TAPS} taps and a positive eps, got {taps}, {eps}")
+        ops.plan_memory_walk(state, value_dim, False, False)  # (refuses memories the walk has no room for)
+        self.hidden_size, self.num_heads, self.value_dim, self.state = hidden_size, num_heads, value_dim, state
+        self.groups, self.taps, self.norm_groups, self.eps = groups, taps, norm_groups, float(eps)
+        self.inner = num_heads * value_dim
+        self.conv_width = self.inner + 2 * groups * state
+
+    def cache_need(self) -> tuple:
+        return (FixedState((self.num_heads, self.state, self.value_dim)),
+                FixedState((max(self.taps - 1, 1), self.conv_width)))
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        small = dict(keeps_float32=True)
+        return {
+            prefix + "in": TensorSpec((2 * self.inner + 2 * self.groups * self.state + self.num_heads, self.hidden_size)),
+            prefix + "conv": TensorSpec((self.conv_width, self.taps)),
+            prefix + "conv.b": TensorSpec((self.conv_width,)),
+            prefix + "dt_bias": TensorSpec((self.num_heads,), **small),
+            prefix + "A_log": TensorSpec((self.num_heads,), **small),
+            prefix + "D": TensorSpec((self.num_heads,), init="norm", **small),
+            prefix + "norm": TensorSpec((self.inner,), init="norm", **small),
+            prefix + "o": TensorSpec((self.hidden_size, self.inner)),
+        }
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        w_in = tensors[prefix + "in"]
+        if w_in.shape[0] % 8:  # (the rows of the product's result stay 16-byte aligned)
+            w_in = torch.cat([w_in, w_in.new_zeros((8 - w_in.shape[0] % 8, self.hidden_size))], dim=0)
+        self.w_in = w_in.contiguous()
+        self.conv_w = tensors[prefix + "conv"].contiguous()
+        self.conv_b = tensors[prefix + "conv.b"].contiguous()
+        self.dt_bias = tensors[prefix + "dt_bias"].float().contiguous()
+        self.a_log = tensors[prefix + "A_log"].float().contiguous()
+        self.skip = tensors[prefix + "D"].float().contiguous()
+        self.norm_weight = tensors[prefix + "norm"].float().contiguous()
+        self.w_o = tensors[prefix + "o"].contiguous()
+
+    def warm_up(self, rows: int) -> None:
+        blank = lambda width: torch.zeros((rows, width), dtype=self.w_in.dtype, device=self.w_in.device)
+        linear(blank(self.hidden_size), self.w_in)
+        linear(blank(self.inner), self.w_o)
+
+    def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+        if not writes:
+            raise ValueError("a recurrent mixer moves its state on whenever it runs")
+        memory, past = view[0].state, view[1].state
+        inner, bc = self.inner, self.groups * self.state
+        proj = linear(x, self.w_in)
+        z, taken, raw_dt = proj[:, :inner], proj[:, inner: inner + self.conv_width], proj[:, 2 * inner + 2 * bc:2 * inner + 2 * bc + self.num_heads]
+        mixed = ops.causal_conv(taken, self.conv_w, self.conv_b, past, batch.seq_of_token, batch.seq_slot,
+                                batch.q_start_loc, activation="silu", out_dtype=torch.float32)
+        ops.conv_keep(taken, past, batch.seq_slot, batch.q_start_loc, batch.sequences, self.taps)
+        steps, decay = ops.space_steps(raw_dt, self.dt_bias, self.a_log)
+        y = ops.memory_walk(decay, mixed[:, inner: inner + bc], mixed[:, inner + bc:], mixed[:, :inner], memory,
+                            batch.seq_slot, batch.q_start_loc, batch.sequences, self.num_heads, self.state,
+                            self.value_dim, heads_per_group=self.num_heads // self.groups, value_scale=steps,
+                            skip=self.skip)
+        out = ops.gated_group_norm(y, z, self.norm_weight, self.norm_groups, self.eps, x.dtype, gate_first=True)
+        return linear(out, self.w_o)
+
+
+class TimeMixing(Part):
+    """Tensors: ``mu.r``, ``mu.k``, ``mu.v``, ``mu.g``, ``mu.w`` [hidden] (how much of the token before each mix takes),
+    ``r``, ``k``, ``v``, ``g`` [heads * dim, hidden], ``w1`` [rank, hidden] and ``w2`` [heads * dim, rank] (the rank is
+    the checkpoint's), ``w0`` [heads * dim], ``u`` [heads, dim], ``norm`` [heads * dim], ``o``.  Mixes and products run
+    in the engine's type; the products' results that enter the memory, decays, the memory, the read-out and its norm
+    are float32."""
+
+    graph_safe = True
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, eps: float, decay_rank: Optional[int] = None) -> None:
+        for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("head_dim", head_dim)):
+            if isinstance(value, bool) or not isinstance(value, int) or value < 1:
+                raise ValueError(f"{name} must be a positive integer, got {value!r}")
+        if not eps > 0:
+            raise ValueError("eps must be positive")
+        ops.plan_memory_walk(head_dim, head_dim, True, True)  # (refuses memories the walk has no room for)
+        self.hidden_size, self.num_heads, self.head_dim, self.eps = hidden_size, num_heads, head_dim, float(eps)
+        self.decay_rank = decay_rank  # None: whatever the checkpoint holds
+        self.channels = num_heads * head_dim
+
+    def cache_need(self) -> tuple:
+        return (FixedState((self.num_heads, self.head_dim, self.head_dim)), FixedState((self.hidden_size,)))
+
+    def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
+        c, hidden = self.channels, self.hidden_size
+        small = dict(keeps_float32=True)
+        drawn_rank = self.decay_rank or max(8, min(64, hidden // 16 // 8 * 8 or 8))
+        out = {prefix + "mu." + name: TensorSpec((hidden,), **small) for name in self.MIXES}
+        out.update({prefix + name: TensorSpec((c, hidden)) for name in ("r", "k", "v", "g")})
+        out[prefix + "w1"] = TensorSpec((self.decay_rank, hidden), drawn=(drawn_rank, hidden))
+        out[prefix + "w2"] = TensorSpec((c, self.decay_rank), drawn=(c, drawn_rank))
+        out[prefix + "w0"] = TensorSpec((c,), **small)
+        out[prefix + "u"] = TensorSpec((self.num_heads, self.head_dim), **small)
+        out[prefix + "norm"] = TensorSpec((c,), init="norm", **small)
+        out[prefix + "o"] = TensorSpec((hidden, c))
+        return out
+
+    def bind(self, tensors, prefix, dtype, device) -> None:
+        super().bind(tensors, prefix, dtype, device)
+        self.mu = torch.stack([tensors[prefix + "mu." + name].float() for name in self.MIXES]).contiguous()
+        self.w_r, self.w_k, self.w_v, self.w_g = (tensors[prefix + name].contiguous() for name in ("r", "k", "v", "g"))
+        self.w_1 = tensors[prefix + "w1"].contiguous()
+        self.w_2 = tensors[prefix + "w2"].contiguous()
+        if self.w_1.shape[0] != self.w_2.shape[1]:
+            raise ValueError(f"{prefix}w1 {tuple(self.w_1.shape)} and {prefix}w2 {tuple(self.w_2.shape)} disagree on the rank")
+        self.w_0 = tensors[prefix + "w0"].float().contiguous()
+        self.bonus = tensors[prefix + "u"].float().contiguous()
+        self.norm_weight = tensors[prefix + "norm"].float().contiguous()
+        self.w_o = tensors[prefix + "o"].contiguous()
+
+    def warm_up(self, rows: int) -> None:
+        blank = lambda width: torch.zeros((rows, width), dtype=self.w_o.dtype, device=self.w_o.device)
+        for weight in (self.w_r, self.w_k, self.w_v, self.w_g):
+            linear(blank(self.hidden_size), weight)
+        linear(blank(self.channels), self.w_o)
+
+    def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+        if not writes:
+            raise ValueError("a recurrent mixer moves its state on whenever it runs")
+        memory, before = view[0].state, view[1].state
+        mixes = ops.shift_mix(x, before, self.mu, batch.seq_of_token, batch.seq_slot, batch.q_start_loc)
+        f32 = torch.float32
+        r = linear(mixes[0], self.w_r, out_dtype=f32)
+        k = linear(mixes[1], self.w_k, out_dtype=f32)
+        v = linear(mixes[2], self.w_v, out_dtype=f32)
+        gate = linear(mixes[3], self.w_g)
+        low = linear(mixes[4], self.w_1, out_dtype=f32)
+        decay = ops.time_decay(low, self.w_2, self.w_0, x, before, batch.seq_of_token, batch.seq_slot, batch.q_start_loc)
+        y = ops.memory_walk(decay, k, r, v, memory, batch.seq_slot, batch.q_start_loc, batch.sequences, self.num_heads,
+                            self.head_dim, self.head_dim, bonus=self.bonus, read_first=True)
+        out = ops.gated_group_norm(y, gate, self.norm_weight, self.num_heads, self.eps, x.dtype, gate_first=False)
+        return linear(out, self.w_o)
+
+
 register_part("mixer", "retention", Retention)
+register_part("mixer", "state_space", StateSpace)
+register_part("mixer", "time_mixing", TimeMixing)
 register_part("mixer", "lightning_attention", LightningAttention)
 register_part("mixer", "gated_linear_recurrence", GatedLinearRecurrence)

@@ -2,12 +2,14 @@
 the position in other ways.  Every step is a parameter of the part and may be left out:
 
 * a per-head RMS norm of queries and keys (``qk_norm``: ``"weight"`` with one weight vector for all query heads
-  and one for all key heads, ``"unit"`` without weights, ``None``);
+  and one for all key heads, ``"unit"`` without weights, ``None``), or (``"whole"``) one RMS norm over all query
+  heads of a token together and one over all its key heads, with a weight for every number of the projection;
 * a factor on the queries that grows with the logarithm of the position (``q_temperature = (coef, every)``:
   ``1 + coef * ln(floor((p + 1) / every) + 1)``);
 * ``score = q . k * scale``, then a smooth cap (``softcap``: ``c * tanh(score / c)``), then a bias on the distance
   itself (``slope_base = b``: head h of H loses ``2^(-b (h + 1) / H) * (i - j)``);
-* a window (``window``: the token itself and the ``window - 1`` before it), or chunks (``chunk``: the token sees the
+* a window (``window``: the token itself and the ``window - 1`` before it; with ``keep_first`` the first that many
+  tokens of the sequence stay visible from behind the window too, at their own positions), or chunks (``chunk``: the token sees the
   keys of its own chunk of that many positions up to itself; chunks are counted from position 0 of the sequence);
 * biases on the projections of queries, keys and values (``qkv_bias``);
 * a rotation of the first numbers of every query and key head by the position (``position``: a position part such
@@ -15,7 +17,9 @@ the position in other ways.  Every step is a parameter of the part and may be le
 * a sink (``sink``: one learned number per head whose exponential stands in the softmax's denominator, and
   nowhere else);
 * a gate on every head's output (``head_gate``: ``sigmoid(W_g x)_h``, read from the layer's own input);
-* key and value heads of different sizes.
+* key and value heads of different sizes;
+* no keys and values of its own (``own_kv=False``): the layer has no tensors for them and reads the cache unit that
+  another layer of the same head sizes writes, with its own queries, mask and everything else.
 
 One product makes queries, keys, values and gate logits; one kernel norms and scales the heads, lays the queries
 out and writes the cache (``ops.heads_prepare``); the attention kernel shapes the scores, and applies sink and
@@ -54,7 +58,8 @@ class ScoredAttention(Part):
                  scale: float, eps: float, window: Optional[int] = None, qk_norm: Optional[str] = None,
                  q_temperature: Optional[tuple] = None, softcap: Optional[float] = None,
                  slope_base: Optional[float] = None, sink: bool = False, head_gate: bool = False,
-                 chunk: Optional[int] = None, qkv_bias: bool = False, position: Optional[PartSpec] = None) -> None:
+                 chunk: Optional[int] = None, qkv_bias: bool = False, position: Optional[PartSpec] = None,
+                 keep_first: int = 0, own_kv: bool = True) -> None:
         for name, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("num_kv_heads", num_kv_heads),
                             ("head_dim", head_dim), ("value_dim", value_dim)):
             if isinstance(value, bool) or not isinstance(value, int) or value < 1:
@@ -67,6 +72,10 @@ class ScoredAttention(Part):
             raise ValueError("window must be positive")
         if chunk is not None and (isinstance(chunk, bool) or not isinstance(chunk, int) or chunk < 1 or window is not None):
             raise ValueError(f"chunks hold a positive number of tokens and stand in a window's place, got {chunk!r}")
+        if isinstance(keep_first, bool) or not isinstance(keep_first, int) or keep_first < 0:
+            raise ValueError(f"keep_first is a count of tokens, got {keep_first!r}")
+        if window is None:
+            keep_first = 0  # (every key is seen anyway)
         if qk_norm not in ops.NORM_MODES:
             raise ValueError(f"qk_norm must be one of {list(ops.NORM_MODES)}, got {qk_norm!r}")
         if not eps > 0:
@@ -84,6 +93,7 @@ class ScoredAttention(Part):
         self.qk_norm, self.q_temperature, self.softcap = qk_norm, q_temperature, softcap
         self.slope_base, self.sink, self.head_gate = slope_base, bool(sink), bool(head_gate)
         self.chunk, self.qkv_bias = chunk, bool(qkv_bias)
+        self.keep_first, self.own_kv = keep_first, bool(own_kv)
         self.position = build_part("position", position) if position is not None else None
         if self.position is not None and self.position.rotates and self.position.rotary_dim > head_dim:
             raise ValueError(f"{self.position.rotary_dim} turning numbers in heads of {head_dim}")
@@ -95,23 +105,25 @@ class ScoredAttention(Part):
     def cache_need(self) -> PagedKV:
         # (a chunk's keys all lie inside a window of the chunk's length: pages behind it go back to the pool)
         return PagedKV(self.num_kv_heads, self.kernel_dim, self.window if self.chunk is None else self.chunk,
-                       value_dim=self.kernel_vdim if self.kernel_vdim != self.kernel_dim else None)
+                       value_dim=self.kernel_vdim if self.kernel_vdim != self.kernel_dim else None,
+                       keep_first=self.keep_first)
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         h, g, d, v, width = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, self.hidden_size
-        out = {
-            prefix + "q": TensorSpec((h * d, width)),
-            prefix + "k": TensorSpec((g * d, width)),
-            prefix + "v": TensorSpec((g * v, width)),
-            prefix + "o": TensorSpec((width, h * v)),
-        }
+        out = {prefix + "q": TensorSpec((h * d, width)), prefix + "o": TensorSpec((width, h * v))}
+        if self.own_kv:
+            out[prefix + "k"] = TensorSpec((g * d, width))
+            out[prefix + "v"] = TensorSpec((g * v, width))
         if self.qkv_bias:
             out[prefix + "q.b"] = TensorSpec((h * d,))
-            out[prefix + "k.b"] = TensorSpec((g * d,))
-            out[prefix + "v.b"] = TensorSpec((g * v,))
-        if self.qk_norm == "weight":
-            out[prefix + "q.norm"] = TensorSpec((d,), init="norm", keeps_float32=True)
-            out[prefix + "k.norm"] = TensorSpec((d,), init="norm", keeps_float32=True)
+            if self.own_kv:
+                out[prefix + "k.b"] = TensorSpec((g * d,))
+                out[prefix + "v.b"] = TensorSpec((g * v,))
+        if self.qk_norm in ("weight", "whole"):
+            whole = self.qk_norm == "whole"
+            out[prefix + "q.norm"] = TensorSpec((h * d if whole else d,), init="norm", keeps_float32=True)
+            if self.own_kv:
+                out[prefix + "k.norm"] = TensorSpec((g * d if whole else d,), init="norm", keeps_float32=True)
         if self.sink:
             out[prefix + "sink"] = TensorSpec((h,), keeps_float32=True)
         if self.head_gate:
@@ -121,14 +133,16 @@ class ScoredAttention(Part):
     def bind(self, tensors, prefix, dtype, device) -> None:
         super().bind(tensors, prefix, dtype, device)
         h, g, d, v = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
-        blocks = [tensors[prefix + "q"], tensors[prefix + "k"], tensors[prefix + "v"]]
-        self.offsets = (0, h * d, h * d + g * d)
+        blocks = [tensors[prefix + "q"]]
+        if self.own_kv:
+            blocks += [tensors[prefix + "k"], tensors[prefix + "v"]]
+        self.offsets = (0, h * d, h * d + g * d) if self.own_kv else (0, 0, 0)
         self.gate_offset = None
         if self.head_gate:
             # gate logits ride in the same product, on columns that start at a multiple of 8 (and the row is
             # padded to one), so that the rows of the result stay 16-byte aligned
             pad = lambda rows: blocks[0].new_zeros((rows, self.hidden_size))
-            used = h * d + g * d + g * v
+            used = h * d + (g * d + g * v if self.own_kv else 0)
             if used % 8:
                 blocks.append(pad(8 - used % 8))
             self.gate_offset = _round8(used)
@@ -138,12 +152,14 @@ class ScoredAttention(Part):
         self.w_in = torch.cat(blocks, dim=0).contiguous()
         self.b_in = None
         if self.qkv_bias:
-            bias = torch.cat([tensors[prefix + "q.b"], tensors[prefix + "k.b"], tensors[prefix + "v.b"]], dim=0)
+            names = ("q.b", "k.b", "v.b") if self.own_kv else ("q.b",)
+            bias = torch.cat([tensors[prefix + name] for name in names], dim=0)
             self.b_in = torch.cat([bias, bias.new_zeros(self.w_in.shape[0] - bias.shape[0])]).contiguous()
         self.q_weight = self.k_weight = None
-        if self.qk_norm == "weight":
+        if self.qk_norm in ("weight", "whole"):
             self.q_weight = tensors[prefix + "q.norm"].float().contiguous()
-            self.k_weight = tensors[prefix + "k.norm"].float().contiguous()
+            if self.own_kv:
+                self.k_weight = tensors[prefix + "k.norm"].float().contiguous()
         self.sinks = tensors[prefix + "sink"].float().contiguous() if self.sink else None
         self.slopes = None
         if self.slope_base is not None:
@@ -162,6 +178,8 @@ class ScoredAttention(Part):
         linear(blank(self.num_heads * self.kernel_vdim), self.w_o)
 
     def forward(self, x: torch.Tensor, batch, view, writes: bool = True) -> torch.Tensor:
+        if writes and not self.own_kv:
+            raise ValueError("a layer without keys and values of its own reads the cache unit that another layer writes")
         proj = linear(x, self.w_in, self.b_in)
         rotary = None
         if self.position is not None and self.position.rotates:
@@ -179,7 +197,7 @@ class ScoredAttention(Part):
 
     def attend(self, q: torch.Tensor, gate, batch, view) -> torch.Tensor:
         shape = dict(window=self.window, scale=self.scale, softcap=self.softcap, slopes=self.slopes,
-                     sinks=self.sinks, gate=gate, chunk=self.chunk)
+                     sinks=self.sinks, gate=gate, chunk=self.chunk, keep_first=self.keep_first)
         h, g = self.num_heads, self.num_kv_heads
         group = h // g
         page_size = view.page_size
@@ -189,6 +207,8 @@ class ScoredAttention(Part):
             # the most keys a token sees in this step (a captured step: in any of its replays)
             bound = batch.static_plan.max_keys if batch.static_plan is not None else batch.max_context
             reach = self.window if self.chunk is None else self.chunk  # the most keys a token sees, if bounded
+            if reach is not None and self.keep_first:
+                reach += -(-self.keep_first // 32) * 32 + 32  # (the kept first keys are walked in whole blocks of 32)
             bound = bound if reach is None else min(bound, reach)
 
             def shares(tiles: int, span: int) -> dict:

@@ -99,7 +99,7 @@ class SafetensorsSource:
         wrong = [
             f"{name}: expected {tuple(spec.shape)}, got {index[name][1]}"
             for name, spec in expected.items()
-            if name in index and tuple(index[name][1]) != tuple(spec.shape)
+            if name in index and not spec.fits(tuple(index[name][1]))
         ]
         if missing or unexpected or wrong:
             raise WeightError(missing, unexpected, wrong)
@@ -176,8 +176,8 @@ class RandomSource:
         generator = torch.Generator(device=self.draw_device)
         generator.manual_seed((self.seed * 1_000_003 + index * 7919 + 12345) % (2**63 - 1))
         if spec.kind == "int":
-            return torch.zeros(spec.shape, dtype=torch.int32, device=self.draw_device)
-        values = torch.randn(spec.shape, generator=generator, dtype=torch.float32,
+            return torch.zeros(spec.random_shape, dtype=torch.int32, device=self.draw_device)
+        values = torch.randn(spec.random_shape, generator=generator, dtype=torch.float32,
                              device=self.draw_device) * self.std
         if spec.init == "norm":
             values += 1.0
