@@ -36,7 +36,7 @@ def softplus(z: torch.Tensor) -> torch.Tensor:
 
 
 def plain_frequencies(dims: int, base: float) -> torch.Tensor:
-    return torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=F)
+    return torch.tensor([base ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=F)  # (angles stay float64)
 
 
 def linear_frequencies(dims: int, base: float, factor: float) -> tuple[torch.Tensor, float]:
@@ -115,9 +115,10 @@ def time_mix_token(memory: torch.Tensor, r: torch.Tensor, k: torch.Tensor, v: to
 
 # ---------------------------------------------------------------------------------------------------- the model
 class Model:
-    def __init__(self, config: dict, tensors: dict) -> None:
+    def __init__(self, config: dict, tensors: dict, dtype: torch.dtype = F) -> None:
         self.config = config
-        self.t = {name: value.to(F) for name, value in tensors.items()}
+        self.dtype = dtype  # float64 is the yardstick; bfloat16 shows what rounding everything to 16 bits costs
+        self.t = {name: value.to(dtype) for name, value in tensors.items()}
         self.eps = float(config["norm"]["eps"])
         self.width = int(config["width"])
         self.layers = config["layers"]
@@ -233,7 +234,7 @@ class Sequence:
         v = (t[p + "v"] @ mix["v"]).reshape(heads, dim)
         gate = silu(t[p + "g"] @ mix["g"])
         w = torch.exp(-torch.exp(t[p + "w2"] @ torch.tanh(t[p + "w1"] @ mix["w"]) + t[p + "w0"])).reshape(heads, dim)
-        memory = self.state.get((index, "memory"), torch.zeros((heads, dim, dim), dtype=F))
+        memory = self.state.get((index, "memory"), torch.zeros((heads, dim, dim), dtype=m.dtype))
         outs, new = [], []
         for i in range(heads):
             s, o = time_mix_token(memory[i], r[i], k[i], v[i], w[i], t[p + "u"][i])
@@ -250,7 +251,7 @@ class Sequence:
         inner = heads * vdim
         proj = t[p + "in"] @ h
         z, xbc, dt = proj[:inner], proj[inner: 2 * inner + 2 * G * N], proj[2 * inner + 2 * G * N:]
-        past = self.state.get((index, "past"), torch.zeros((taps - 1, xbc.shape[0]), dtype=F))
+        past = self.state.get((index, "past"), torch.zeros((taps - 1, xbc.shape[0]), dtype=m.dtype))
         inputs = torch.cat([past, xbc[None]], dim=0)                         # the last `taps` inputs, oldest first
         xbc = silu((inputs * t[p + "conv"].t()).sum(0) + t[p + "conv.b"])
         self.state[(index, "past")] = inputs[1:]
@@ -258,7 +259,7 @@ class Sequence:
         b = xbc[inner: inner + G * N].reshape(G, N)
         cc = xbc[inner + G * N:].reshape(G, N)
         dt = softplus(dt + t[p + "dt_bias"])
-        memory = self.state.get((index, "memory"), torch.zeros((heads, N, vdim), dtype=F))
+        memory = self.state.get((index, "memory"), torch.zeros((heads, N, vdim), dtype=m.dtype))
         ys, new = [], []
         for i in range(heads):
             g = i // (heads // G)
@@ -284,3 +285,8 @@ class Sequence:
             shared = gated_unit(h, t[p + "shared.gate"], t[p + "shared.up"], t[p + "shared.down"], silu)
             out = out + torch.sigmoid(t[p + "shared.sg"] @ h)[0] * shared
         return out
+
+
+def forward(config: dict, tensors: dict, tokens, dtype: torch.dtype = F) -> torch.Tensor:
+    """Logits [len(tokens), vocab] of one sequence from its start."""
+    return Model(config, tensors, dtype).logits(tokens)
