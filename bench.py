@@ -5,7 +5,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096]
                     [--shape 0.5b|3b|7b|14b|32b|72b] [--layers N] [--long-contexts 32768]
                     [--mixed-portions 16,64,248] [--other-shapes 7b,14b]
-    python bench.py --design polosun|givizen|nokipel [--design-shapes 3b,7b] [--design-layers 12]
+    python bench.py --design polosun|givizen|nokipel|senuvik [--design-shapes 3b,7b] [--design-layers 12]
 
 A "step" is one decode step of the whole engine (scheduler iteration: plan,
 step function, sampling, token hand-over).  Protocol after the reference's
@@ -44,7 +44,13 @@ layers of lightning attention to one of chunked softmax attention, dense
 bounded feed-forwards and routed experts in turn) beside the Givizen model of
 equal width, head sizes, expert sizes, vocabulary and layer count, the closest
 of the engine's models: the same attention and expert kernels with other
-options.
+options.  ``--design senuvik`` measures the Senuvik design (window attention
+with kept first tokens, a state-space mixer, causal attention beside time
+mixing, and window attention on another layer's keys in turn; a dense
+feed-forward and routed experts) beside the Nokipel model of equal width, head
+sizes, expert sizes, vocabulary and layer count, the closest of the engine's
+models: memories of fixed size beside attention, dense and routed
+feed-forwards.
 """
 
 from __future__ import annotations
@@ -410,11 +416,113 @@ def nokipel_costs(config, batch: int, context: float, tokens: int, elem: int) ->
     return moved, flops
 
 
+SENUVIK_WINDOW, SENUVIK_KEPT = 1024, 64
+
+
+def senuvik_raw(shape: dict, layers: int) -> dict:
+    """A Senuvik configuration with the width, vocabulary, head counts and head size of a Qwen2.5 shape.  Of every
+    four layers the first has window attention (1,024 tokens beside 64 kept first ones, a rotation over half of each
+    head) and a dense feed-forward of the shape's size, the second a state-space mixer twice as wide as the stream
+    (heads of 64 numbers, memories of 128 rows, 8 groups), the third causal attention beside time mixing (heads of
+    64), and the fourth window attention on the first layer's keys and values; these three have routed feed-forwards
+    of Givizen's sizes (32 experts, 4 per token, a gated shared expert)."""
+    width = shape["hidden_size"]
+    heads, kv_heads = shape["num_attention_heads"], shape["num_key_value_heads"]
+    dim = width // heads
+    expert_ff = shape["intermediate_size"] // (2 * GIVIZEN_TOP) // 64 * 64
+    shared_ff = shape["intermediate_size"] - GIVIZEN_TOP * expert_ff
+    dense = {"kind": "dense", "ff": shape["intermediate_size"]}
+    routed = {"kind": "moe", "expert": {"ff": expert_ff}, "shared": {"ff": shared_ff},
+              "router": {"experts": GIVIZEN_EXPERTS, "top": GIVIZEN_TOP}}
+    window = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+              "mask": {"size": SENUVIK_WINDOW, "keep_first": SENUVIK_KEPT},
+              "rot": {"base": 1000000.0, "dims": dim // 2, "scaling": {"factor": 4.0}}}
+    space = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}
+    pair = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "softcap": 50.0,
+                     "rot": {"base": 1000000.0, "dims": dim,
+                             "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+            "right": {"heads": width // 64, "dim": 64}, "left_scale": 0.5, "right_scale": 0.5}
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        if kind == 0:
+            out.append({"type": "attention", "mixer": dict(window), "mlp": dense})
+        elif kind == 1:
+            out.append({"type": "mamba2", "mixer": space, "mlp": routed})
+        elif kind == 2:
+            out.append({"type": "parallel", "mixer": pair, "mlp": routed})
+        else:
+            out.append({"type": "attention", "mixer": dict(window, kv_from=i - 3), "mlp": routed})
+    return {"architecture": "Senuvik", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6}, "layers": out}
+
+
+SENUVIK_DECAY_RANK = 64   # (the rank of the decay's two small products is the checkpoint's; random weights draw this)
+
+
+def senuvik_costs(config, batch: int, context: float, tokens: int, elem: int) -> tuple[float, float]:
+    """(bytes one decode step has to move, flops of a prefill of ``tokens`` tokens) for a Senuvik configuration:
+    every weight that a step touches once (of a layer's experts, the ones that ``batch`` tokens choosing ``top`` of
+    them at random are expected to hit), each request's keys and values inside the window and among the kept first
+    tokens (once for the layer that writes them and once for every layer that reads them), every memory read and
+    written in float32; products at two flops per active weight and token, attention over the keys a token sees,
+    the memories' updates and read-outs."""
+    width, vocab = config.hidden_size, config.vocab_size
+    moved = float(vocab * width * elem)
+    flops = 2.0 * vocab * width
+
+    def attention(m, size, keep):
+        nonlocal moved, flops
+        seen = context if size is None else min(context, size + keep)
+        moved += batch * seen * m["kv_heads"] * (m["dim"] + m["vdim"]) * elem
+        if size is None:
+            pairs = tokens * (tokens + 1) / 2
+        else:
+            reach = min(tokens, size)
+            pairs = reach * (reach + 1) / 2 + (tokens - reach) * (reach + keep)
+        flops += 2.0 * pairs * m["heads"] * (m["dim"] + m["vdim"])
+
+    for layer in config.raw["layers"]:
+        m, mlp = layer["mixer"], layer["mlp"]
+        if layer["type"] == "attention":
+            own = m.get("kv_from") is None
+            mixer = width * (m["heads"] * m["dim"] + m["heads"] * m["vdim"])
+            mixer += width * m["kv_heads"] * (m["dim"] + m["vdim"]) if own else 0
+            attention(m, m["mask"]["size"], m["mask"].get("keep_first", 0))
+        elif layer["type"] == "mamba2":
+            inner = m["heads"] * m["vdim"]
+            mixer = width * (2 * inner + 2 * m["groups"] * m["state"] + m["heads"]) + inner * width
+            moved += batch * 2 * m["heads"] * m["state"] * m["vdim"] * 4
+            flops += 2.0 * 2 * tokens * m["heads"] * m["state"] * m["vdim"]
+        else:
+            left, right = m["left"], m["right"]
+            mixer = width * (left["heads"] * left["dim"] + left["kv_heads"] * (left["dim"] + left["vdim"])
+                             + left["heads"] * left["vdim"] + left["heads"])
+            channels = right["heads"] * right["dim"]
+            mixer += 5 * width * channels + SENUVIK_DECAY_RANK * (width + channels)
+            attention(left, None, 0)
+            moved += batch * 2 * right["heads"] * right["dim"] * right["dim"] * 4
+            flops += 2.0 * 2 * tokens * right["heads"] * right["dim"] * right["dim"]
+        if mlp is None:
+            active = touched = 0.0
+        elif mlp["kind"] == "dense":
+            active = touched = 3.0 * width * mlp["ff"]
+        else:
+            experts, top = mlp["router"]["experts"], mlp["router"]["top"]
+            one = 3 * width * mlp["expert"]["ff"]
+            shared = 3 * width * mlp["shared"]["ff"] + width if mlp.get("shared") else 0
+            hit = experts * (1.0 - (1.0 - top / experts) ** batch)
+            touched = width * experts + shared + hit * one
+            active = width * experts + shared + top * one
+        moved += (mixer + touched) * elem
+        flops += 2.0 * tokens * (mixer + active)
+    return moved, flops
+
+
 def compare_designs(args) -> int:
-    """``--design polosun``, ``--design givizen`` or ``--design nokipel``: see the module's text."""
+    """``--design polosun``, ``--design givizen``, ``--design nokipel`` or ``--design senuvik``: see the module's text."""
     import torch
 
-    from cie_amd.config import GivizenConfig, NokipelConfig, PolosunConfig, Qwen2Config
+    from cie_amd.config import GivizenConfig, NokipelConfig, PolosunConfig, Qwen2Config, SenuvikConfig
     from cie_amd.workloads import SHAPES
 
     elem = 2 if args.dtype == "bf16" else 4
@@ -425,6 +533,9 @@ def compare_designs(args) -> int:
         if args.design == "nokipel":
             designs = {"nokipel": NokipelConfig.from_hf_config(nokipel_raw(shape, layers)),
                        "givizen": GivizenConfig.from_hf_config(givizen_raw(shape, layers))}
+        elif args.design == "senuvik":
+            designs = {"senuvik": SenuvikConfig.from_hf_config(senuvik_raw(shape, layers)),
+                       "nokipel": NokipelConfig.from_hf_config(nokipel_raw(shape, layers))}
         else:
             designs = {
                 args.design: (PolosunConfig.from_hf_config(polosun_raw(shape, layers)) if args.design == "polosun"
@@ -440,6 +551,8 @@ def compare_designs(args) -> int:
                     return givizen_costs(config, batch, context, args.prefill_tokens, elem)
                 if design == "nokipel":
                     return nokipel_costs(config, batch, context, args.prefill_tokens, elem)
+                if design == "senuvik":
+                    return senuvik_costs(config, batch, context, args.prefill_tokens, elem)
                 return (decode_bytes(config, layers, batch, context, elem), prefill_flops(config, layers, args.prefill_tokens))
 
             record = {}
@@ -465,7 +578,15 @@ def compare_designs(args) -> int:
             out[name][design] = record
     givizen_layers = (f"attention (window {GIVIZEN_WINDOWS[0]}) and attention_2 (window {GIVIZEN_WINDOWS[1]}) in turn, each "
                       f"with {GIVIZEN_EXPERTS} experts, {GIVIZEN_TOP} per token, and a shared expert")
+    nokipel_layers = (f"lightning + dense, lightning + experts, lightning + dense, attention (chunks of "
+                      f"{GIVIZEN_WINDOWS[0]}) + experts in turn; {GIVIZEN_EXPERTS - NOKIPEL_IDENTITY} experts and "
+                      f"{NOKIPEL_IDENTITY} identity experts in {NOKIPEL_GROUPS[0]} groups ({NOKIPEL_GROUPS[1]} kept), "
+                      f"{GIVIZEN_TOP} per token, and a gated shared expert")
+    senuvik_layers = (f"window attention ({SENUVIK_WINDOW} tokens beside {SENUVIK_KEPT} kept first ones) + dense, state space + "
+                      f"experts, causal attention beside time mixing + experts, window attention on the first layer's keys "
+                      f"+ experts in turn; {GIVIZEN_EXPERTS} experts, {GIVIZEN_TOP} per token, and a gated shared expert")
     beside = ("the Givizen model of equal width, head and expert sizes" if args.design == "nokipel"
+              else "the Nokipel model of equal width, head and expert sizes" if args.design == "senuvik"
               else "the Qwen2.5 decoder of equal width, feed-forward")
     print(json.dumps({
         "metric": f"{args.design.capitalize()} beside {beside}, vocabulary and {layers} layers",
@@ -474,10 +595,8 @@ def compare_designs(args) -> int:
         "config": {"layers": layers, "context": args.context, "prefill_tokens": args.prefill_tokens, "page_size": PAGE,
                    "design_layers": ("retention, latent_attention, rglru in turn, each with a dense feed-forward"
                                      if args.design == "polosun" else givizen_layers if args.design == "givizen" else
-                                     f"lightning + dense, lightning + experts, lightning + dense, attention (chunks of "
-                                     f"{GIVIZEN_WINDOWS[0]}) + experts in turn; {GIVIZEN_EXPERTS - NOKIPEL_IDENTITY} experts and "
-                                     f"{NOKIPEL_IDENTITY} identity experts in {NOKIPEL_GROUPS[0]} groups ({NOKIPEL_GROUPS[1]} kept), "
-                                     f"{GIVIZEN_TOP} per token, and a gated shared expert; beside it Givizen: " + givizen_layers)},
+                                     senuvik_layers + "; beside it Nokipel: " + nokipel_layers if args.design == "senuvik" else
+                                     nokipel_layers + "; beside it Givizen: " + givizen_layers)},
         "shapes": out,
     }))
     return 0
@@ -504,9 +623,9 @@ def main(argv=None) -> int:
                              "(default 16,64,248; '' for none, as with --no-points)")
     parser.add_argument("--other-shapes", default="7b,14b",
                         help="further shapes whose decode at the main batch and context and whose prefill go into the points ('' for none)")
-    parser.add_argument("--design", default=None, choices=["polosun", "givizen", "nokipel"],
+    parser.add_argument("--design", default=None, choices=["polosun", "givizen", "nokipel", "senuvik"],
                         help="instead of the default record: this design beside the Qwen2.5 decoder of equal size "
-                             "(nokipel: beside the Givizen model of equal size)")
+                             "(nokipel: beside the Givizen model of equal size; senuvik: beside the Nokipel model)")
     parser.add_argument("--design-shapes", default="3b,7b", help="the Qwen2.5 shapes whose sizes the comparison takes")
     parser.add_argument("--design-layers", type=int, default=12, help="layers of both models in the comparison")
     args = parser.parse_args(argv)

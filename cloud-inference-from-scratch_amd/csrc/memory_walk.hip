@@ -21,16 +21,14 @@ __device__ __forceinline__ float silu_f(float x) { return x * sigmoid_f(x); }
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 
 struct WalkArgs {
-    const float* decay;   // decay[t * ld_decay + head * decay_head_stride + n * decay_row_stride]  (row stride 0: one per head)
+    const float* decay;   // a decay per row: decay[t * ld_decay + head * rows + n]; one per head: decay[t * ld_decay + head]
     long ld_decay;
-    int decay_head_stride;
-    int decay_row_stride;
     const float* in;      // in[t * ld_in + (head / heads_per_group) * rows + n]
     long ld_in;
     const float* out;     // out[t * ld_out + (head / heads_per_group) * rows + n]
     long ld_out;
     int heads_per_group;
-    const float* bonus;   // [heads, rows] or null; with read_first only
+    const float* bonus;   // [heads, rows] or null; with the read-out in front of the update only
     const float* val;     // val[t * ld_val + head * cols + p]
     long ld_val;
     const float* val_scale;  // val_scale[t * ld_scale + head] or null: the update takes val * scale
@@ -40,31 +38,36 @@ struct WalkArgs {
     const int* seq_slot;
     const int* q_start_loc;
     float* y;             // [tokens, heads * cols]
-    int heads, rows, cols, slice, row_groups, chunk, read_first;
+    int heads, rows, cols, slice, row_groups, chunk;
 };
 
 // One workgroup per (sequence, head, slice of columns).  Thread (column, row group g) keeps rows g * NS .. + NS - 1
 // of its column in registers.  Tokens go in chunks: the chunk's row operands are staged in LDS (a row group's numbers
-// NS + 4 floats apart from the next group's, so that the groups of a wave read different banks), every thread walks
-// the chunk's tokens in order, and the row groups' shares of y meet in LDS behind the chunk.  The order of every sum
-// depends on the sizes alone, never on what else the step holds.
-template <int NS>
+// NS + 4 floats apart from the next group's, so that the groups of a wave read different banks, and every group's
+// numbers start at a multiple of 16 bytes: a thread reads them four at a time), every thread walks the chunk's tokens
+// in order, the next token's operands on their way from LDS while this token's are worked on, and the row groups'
+// shares of y meet in LDS behind the chunk.  The order of every sum depends on the sizes alone, never on what else
+// the step holds.  TIME: a decay per row, the read-out in front of the update, a bonus; else one decay per head and
+// token, the read-out behind the update.
+template <int NS, bool TIME>
 __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
-    extern __shared__ float lds[];
+    extern __shared__ float4 lds4[];
+    float* lds = reinterpret_cast<float*>(lds4);
+    constexpr int Q = NS / 4;
     const int seq = blockIdx.x;
     const int head = blockIdx.y;
     const int col0 = blockIdx.z * a.slice;
     const int RG = a.row_groups;
     const int pitch = NS + 4;
     const int per_token = RG * pitch;
-    const bool per_row_decay = a.decay_row_stride != 0;
+    const int chunk4 = (a.chunk + 3) & ~3;
     float* in_s = lds;                                   // [chunk][RG][pitch]
     float* out_s = in_s + a.chunk * per_token;           // [chunk][RG][pitch]
-    float* dec_s = out_s + a.chunk * per_token;          // [chunk][RG][pitch] (a decay per row) or [chunk]
-    float* bon_s = dec_s + (per_row_decay ? a.chunk * per_token : a.chunk);  // [chunk][RG][pitch] with a bonus
-    float* val_s = bon_s + (a.bonus ? a.chunk * per_token : 0);              // [chunk][slice]
+    float* dec_s = out_s + a.chunk * per_token;          // TIME: [chunk][RG][pitch]; else [chunk]
+    float* bon_s = dec_s + (TIME ? a.chunk * per_token : chunk4);  // TIME: [chunk][RG][pitch]
+    float* val_s = bon_s + (TIME ? a.chunk * per_token : 0);       // [chunk][slice]
     float* scl_s = val_s + a.chunk * a.slice;            // [chunk]
-    float* part_s = scl_s + a.chunk;                     // [chunk][RG][slice]
+    float* part_s = scl_s + chunk4;                      // [chunk][RG][slice]
 
     const int col = threadIdx.x % a.slice;
     const int rg = threadIdx.x / a.slice;
@@ -92,9 +95,10 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
             const float x = real ? a.in[token * a.ld_in + group * a.rows + n] : 0.f;
             in_s[at] = x;
             out_s[at] = real ? a.out[token * a.ld_out + group * a.rows + n] : 0.f;
-            if (per_row_decay)
-                dec_s[at] = real ? a.decay[token * a.ld_decay + head * a.decay_head_stride + n * a.decay_row_stride] : 0.f;
-            if (a.bonus) bon_s[at] = real ? a.bonus[head * a.rows + n] * x : 0.f;
+            if (TIME) {
+                dec_s[at] = real ? a.decay[token * a.ld_decay + head * a.rows + n] : 0.f;
+                bon_s[at] = (real && a.bonus) ? a.bonus[head * a.rows + n] * x : 0.f;
+            }
         }
         for (int idx = threadIdx.x; idx < n_tok * a.slice; idx += blockDim.x) {
             const int t = idx / a.slice;
@@ -105,41 +109,75 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
         for (int t = threadIdx.x; t < n_tok; t += blockDim.x) {
             const size_t token = static_cast<size_t>(first + from + t);
             scl_s[t] = a.val_scale ? a.val_scale[token * a.ld_scale + head] : 1.f;
-            if (!per_row_decay) dec_s[t] = a.decay[token * a.ld_decay + head * a.decay_head_stride];
+            if (!TIME) dec_s[t] = a.decay[token * a.ld_decay + head];
         }
         __syncthreads();
         if (rg < RG) {
+            const int base = rg * pitch;
+            float4 in_next[Q], out_next[Q], dec_next[TIME ? Q : 1], bon_next[TIME ? Q : 1];
+            float v_next = val_s[col] * scl_s[0];
+            float d_next = TIME ? 0.f : dec_s[0];
+#pragma unroll
+            for (int r = 0; r < Q; ++r) {
+                in_next[r] = reinterpret_cast<const float4*>(in_s + base)[r];
+                out_next[r] = reinterpret_cast<const float4*>(out_s + base)[r];
+                if (TIME) {
+                    dec_next[r] = reinterpret_cast<const float4*>(dec_s + base)[r];
+                    bon_next[r] = reinterpret_cast<const float4*>(bon_s + base)[r];
+                }
+            }
             for (int t = 0; t < n_tok; ++t) {
-                const float* in_t = in_s + t * per_token + rg * pitch;
-                const float* out_t = out_s + t * per_token + rg * pitch;
-                const float raw = val_s[t * a.slice + col];
-                const float v = raw * scl_s[t];
-                float acc = 0.f;
-                if (a.read_first) {
-                    const float* dec_t = dec_s + t * per_token + rg * pitch;
-                    const float* bon_t = bon_s + t * per_token + rg * pitch;
+                float4 in_now[Q], out_now[Q], dec_now[TIME ? Q : 1], bon_now[TIME ? Q : 1];
+                const float v = v_next;
+                const float d = d_next;
 #pragma unroll
-                    for (int i = 0; i < NS; ++i) {
-                        const float bonus = a.bonus ? bon_t[i] : 0.f;
-                        acc = fmaf(out_t[i], fmaf(bonus, v, S[i]), acc);
-                        S[i] = fmaf(per_row_decay ? dec_t[i] : dec_s[t], S[i], in_t[i] * v);
-                    }
-                } else if (per_row_decay) {
-                    const float* dec_t = dec_s + t * per_token + rg * pitch;
-#pragma unroll
-                    for (int i = 0; i < NS; ++i) {
-                        S[i] = fmaf(dec_t[i], S[i], in_t[i] * v);
-                        acc = fmaf(out_t[i], S[i], acc);
-                    }
-                } else {
-                    const float d = dec_s[t];
-#pragma unroll
-                    for (int i = 0; i < NS; ++i) {
-                        S[i] = fmaf(d, S[i], in_t[i] * v);
-                        acc = fmaf(out_t[i], S[i], acc);
+                for (int r = 0; r < Q; ++r) {
+                    in_now[r] = in_next[r];
+                    out_now[r] = out_next[r];
+                    if (TIME) {
+                        dec_now[r] = dec_next[r];
+                        bon_now[r] = bon_next[r];
                     }
                 }
-                part_s[(t * RG + rg) * a.slice + col] = acc;
+                const int ahead = min(t + 1, n_tok - 1);  // (the last token is read twice: no condition around the reads)
+                const int at = ahead * per_token + base;
+                v_next = val_s[ahead * a.slice + col] * scl_s[ahead];
+                if (!TIME) d_next = dec_s[ahead];
+#pragma unroll
+                for (int r = 0; r < Q; ++r) {
+                    in_next[r] = reinterpret_cast<const float4*>(in_s + at)[r];
+                    out_next[r] = reinterpret_cast<const float4*>(out_s + at)[r];
+                    if (TIME) {
+                        dec_next[r] = reinterpret_cast<const float4*>(dec_s + at)[r];
+                        bon_next[r] = reinterpret_cast<const float4*>(bon_s + at)[r];
+                    }
+                }
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll
+                for (int r = 0; r < Q; ++r) {
+                    const float4 k4 = in_now[r], q4 = out_now[r];
+                    if (TIME) {
+                        const float4 w4 = dec_now[r], b4 = bon_now[r];
+                        a0 = fmaf(q4.x, fmaf(b4.x, v, S[4 * r + 0]), a0);
+                        a1 = fmaf(q4.y, fmaf(b4.y, v, S[4 * r + 1]), a1);
+                        a2 = fmaf(q4.z, fmaf(b4.z, v, S[4 * r + 2]), a2);
+                        a3 = fmaf(q4.w, fmaf(b4.w, v, S[4 * r + 3]), a3);
+                        S[4 * r + 0] = fmaf(w4.x, S[4 * r + 0], k4.x * v);
+                        S[4 * r + 1] = fmaf(w4.y, S[4 * r + 1], k4.y * v);
+                        S[4 * r + 2] = fmaf(w4.z, S[4 * r + 2], k4.z * v);
+                        S[4 * r + 3] = fmaf(w4.w, S[4 * r + 3], k4.w * v);
+                    } else {
+                        S[4 * r + 0] = fmaf(d, S[4 * r + 0], k4.x * v);
+                        S[4 * r + 1] = fmaf(d, S[4 * r + 1], k4.y * v);
+                        S[4 * r + 2] = fmaf(d, S[4 * r + 2], k4.z * v);
+                        S[4 * r + 3] = fmaf(d, S[4 * r + 3], k4.w * v);
+                        a0 = fmaf(q4.x, S[4 * r + 0], a0);
+                        a1 = fmaf(q4.y, S[4 * r + 1], a1);
+                        a2 = fmaf(q4.z, S[4 * r + 2], a2);
+                        a3 = fmaf(q4.w, S[4 * r + 3], a3);
+                    }
+                }
+                part_s[(t * RG + rg) * a.slice + col] = (a0 + a1) + (a2 + a3);
             }
         }
         __syncthreads();
@@ -273,39 +311,45 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
 
 }  // namespace
 
-// The walk (see the head of this file).  `rows_per_thread` in {8, 16, 32, 64}; `row_groups * rows_per_thread >= rows`;
-// `slice` columns a workgroup, `slice * row_groups <= 512` threads; `chunk` tokens staged at once.
-CIE_API int cie_memory_walk(void* stream, const float* decay, long ld_decay, int decay_head_stride, int decay_row_stride,
-                            const float* in, long ld_in, const float* out, long ld_out, int heads_per_group,
-                            const float* bonus, const float* val, long ld_val, const float* val_scale, long ld_scale,
-                            const float* skip, float* state, const int* seq_slot, const int* q_start_loc, float* y,
-                            int sequences, int heads, int rows, int cols, int rows_per_thread, int row_groups, int slice,
-                            int chunk, int read_first) {
+// The walk (see the head of this file).  `time_form`: a decay per row ([tokens, heads * rows]), the read-out in front of
+// the update, `bonus` if given; else one decay per head and token ([tokens, heads]) and the read-out behind the update.
+// `rows_per_thread` in {4, 8, 16, 32, 64}; `row_groups * rows_per_thread >= rows`; `slice` columns a workgroup,
+// `slice * row_groups <= 512` threads; `chunk` tokens staged at once.
+CIE_API int cie_memory_walk(void* stream, const float* decay, long ld_decay, const float* in, long ld_in,
+                            const float* out, long ld_out, int heads_per_group, const float* bonus, const float* val,
+                            long ld_val, const float* val_scale, long ld_scale, const float* skip, float* state,
+                            const int* seq_slot, const int* q_start_loc, float* y, int sequences, int heads, int rows,
+                            int cols, int rows_per_thread, int row_groups, int slice, int chunk, int time_form) {
     if (sequences < 0 || heads <= 0 || heads > 65535 || rows <= 0 || cols <= 0 || heads_per_group <= 0 ||
         heads % heads_per_group || row_groups <= 0 || slice <= 0 || chunk <= 0 ||
         static_cast<long>(rows_per_thread) * row_groups < rows || slice * row_groups > 512 || !decay || !in || !out ||
-        !val || !state || !y || (bonus && !read_first))
+        !val || !state || !y || (bonus && !time_form))
         return CIE_BAD_ARGUMENT;
     const int slices = (cols + slice - 1) / slice;
     if (slices > 65535) return CIE_BAD_ARGUMENT;
     const int per_token = row_groups * (rows_per_thread + 4);
-    const size_t floats = static_cast<size_t>(chunk) *
-                              (2 * per_token + (decay_row_stride ? per_token : 1) + (bonus ? per_token : 0) + slice + 1 +
-                               static_cast<size_t>(row_groups) * slice);
+    const int chunk4 = (chunk + 3) & ~3;
+    const size_t floats = static_cast<size_t>(chunk) * ((time_form ? 4 : 2) * per_token + slice +
+                                                        static_cast<size_t>(row_groups) * slice) +
+                          (time_form ? 1 : 2) * chunk4;
     if (floats * sizeof(float) > 64 * 1024) return CIE_BAD_ARGUMENT;
     if (sequences == 0) return CIE_OK;
-    WalkArgs a{decay, ld_decay, decay_head_stride, decay_row_stride, in, ld_in, out, ld_out, heads_per_group, bonus,
-               val, ld_val, val_scale, ld_scale, skip, state, seq_slot, q_start_loc, y, heads, rows, cols, slice,
-               row_groups, chunk, read_first};
+    WalkArgs a{decay, ld_decay, in, ld_in, out, ld_out, heads_per_group, bonus, val, ld_val, val_scale, ld_scale,
+               skip, state, seq_slot, q_start_loc, y, heads, rows, cols, slice, row_groups, chunk};
     const int threads = ((slice * row_groups + kWave - 1) / kWave) * kWave;
     const dim3 grid(sequences, heads, slices);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t lds = floats * sizeof(float);
-    if (rows_per_thread == 8) memory_walk_kernel<8><<<grid, threads, lds, s>>>(a);
-    else if (rows_per_thread == 16) memory_walk_kernel<16><<<grid, threads, lds, s>>>(a);
-    else if (rows_per_thread == 32) memory_walk_kernel<32><<<grid, threads, lds, s>>>(a);
-    else if (rows_per_thread == 64) memory_walk_kernel<64><<<grid, threads, lds, s>>>(a);
+#define CIE_WALK(NS)                                                                       \
+    if (time_form) memory_walk_kernel<NS, true><<<grid, threads, lds, s>>>(a);              \
+    else memory_walk_kernel<NS, false><<<grid, threads, lds, s>>>(a)
+    if (rows_per_thread == 4) { CIE_WALK(4); }
+    else if (rows_per_thread == 8) { CIE_WALK(8); }
+    else if (rows_per_thread == 16) { CIE_WALK(16); }
+    else if (rows_per_thread == 32) { CIE_WALK(32); }
+    else if (rows_per_thread == 64) { CIE_WALK(64); }
     else return CIE_BAD_ARGUMENT;
+#undef CIE_WALK
     return cie_after_launch();
 }
 

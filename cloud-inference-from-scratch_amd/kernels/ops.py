@@ -1131,30 +1131,29 @@ def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, g
 
 
 # ---------------------------------------------------------------------------
-WALK_ROWS = (8, 16, 32, 64)   # rows of a memory that one thread of the walk keeps in registers
+WALK_ROWS = (4, 8, 16, 32, 64)   # rows of a memory that one thread of the walk keeps in registers
 WALK_MAX_ROWS = 1024
 WALK_LDS_BYTES = 48 * 1024
 
 
-def plan_memory_walk(rows: int, cols: int, per_row_decay: bool, bonus: bool, units: int = 1) -> tuple[int, int, int, int]:
+def plan_memory_walk(rows: int, cols: int, time_form: bool, units: int = 1) -> tuple[int, int, int, int]:
     """(rows per thread, row groups, columns per workgroup, tokens staged at once) of ``memory_walk`` for a memory
     of ``rows`` x ``cols`` per head, of which ``units`` (sequences x heads) are walked at once.  Rows per thread and
-    row groups follow from ``rows`` alone (they fix the order of the read-out's sums); the columns are cut into more
+    row groups follow from ``rows`` alone (they fix the order of the read-out's sums): few rows a thread, so that a
+    prompt of one sequence still brings several waves to every compute unit.  The columns are cut into more
     workgroups while these are fewer than the compute units."""
     if not (1 <= rows <= WALK_MAX_ROWS and cols >= 1):
         raise ValueError(f"a memory of {rows} x {cols}: up to {WALK_MAX_ROWS} rows")
-    per_thread = 8 if rows <= 8 else 16 if rows <= 64 else 32 if rows <= 256 else 64
+    per_thread = next(n for n in WALK_ROWS if 16 * n >= rows)
     groups = -(-rows // per_thread)
-    widest = 1 << (min(cols, 64, 512 // groups) - 1).bit_length()  # (a power of two that holds the columns, at most 64)
-    widest = min(widest, 64)
-    while widest * groups > 512:
-        widest //= 2
-    slice_cols = widest
-    while slice_cols > 16 and units * -(-cols // slice_cols) < compute_units():
+    slice_cols = 16
+    while slice_cols < min(cols, 64) and 2 * slice_cols * groups <= 512:
+        slice_cols *= 2
+    while slice_cols > 16 and units * -(-cols // slice_cols) < 2 * compute_units():
         slice_cols //= 2
     per_token = groups * (per_thread + 4)
-    floats = 2 * per_token + (per_token if per_row_decay else 1) + (per_token if bonus else 0) + slice_cols + 1 + groups * slice_cols
-    chunk = max(1, min(16, WALK_LDS_BYTES // (4 * floats)))
+    floats = (4 if time_form else 2) * per_token + slice_cols + groups * slice_cols
+    chunk = max(1, min(16, (WALK_LDS_BYTES - 64) // (4 * floats)))
     return per_thread, groups, slice_cols, chunk
 
 
@@ -1174,7 +1173,7 @@ def memory_walk(decay: torch.Tensor, in_rows: torch.Tensor, out_rows: torch.Tens
     groups_of_heads = heads // heads_per_group
     if heads % heads_per_group:
         raise ValueError(f"{heads} heads in groups of {heads_per_group}")
-    per_row = decay.dim() == 2 and decay.shape[1] == heads * rows and rows > 1
+    per_row = bool(read_first)  # (the read-out in front of the update comes with a decay per row, the other form with one per head)
     for name, t, width in (("decay", decay, heads * rows if per_row else heads), ("in_rows", in_rows, groups_of_heads * rows),
                            ("out_rows", out_rows, groups_of_heads * rows), ("values", values, heads * cols)):
         if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1 and tuple(t.shape) == (tokens, width)):
@@ -1200,14 +1199,14 @@ def memory_walk(decay: torch.Tensor, in_rows: torch.Tensor, out_rows: torch.Tens
         _gpu(name, meta, torch.int32, 1)
         if meta.shape[0] < least:
             raise ValueError(f"{name} has {meta.shape[0]} entries for {sequences} sequences")
-    per_thread, row_groups, slice_cols, chunk = plan_memory_walk(rows, cols, per_row, bonus is not None, sequences * heads)
+    per_thread, row_groups, slice_cols, chunk = plan_memory_walk(rows, cols, per_row, sequences * heads)
     y = torch.empty((tokens, heads * cols), dtype=torch.float32, device=values.device)
     ld = lambda t: t.stride(0) if tokens > 1 else max(t.stride(0), t.shape[1])
     _run("cie_memory_walk", load_library().cie_memory_walk(
-        _stream(), _ptr(decay), ld(decay), _i(rows if per_row else 1), _i(1 if per_row else 0), _ptr(in_rows), ld(in_rows),
-        _ptr(out_rows), ld(out_rows), _i(heads_per_group), _ptr(bonus), _ptr(values), ld(values), _ptr(value_scale),
-        ld_scale, _ptr(skip), _ptr(state), _ptr(seq_slot), _ptr(q_start_loc), _ptr(y), _i(sequences), _i(heads), _i(rows),
-        _i(cols), _i(per_thread), _i(row_groups), _i(slice_cols), _i(chunk), _i(1 if read_first else 0)))
+        _stream(), _ptr(decay), ld(decay), _ptr(in_rows), ld(in_rows), _ptr(out_rows), ld(out_rows), _i(heads_per_group),
+        _ptr(bonus), _ptr(values), ld(values), _ptr(value_scale), ld_scale, _ptr(skip), _ptr(state), _ptr(seq_slot),
+        _ptr(q_start_loc), _ptr(y), _i(sequences), _i(heads), _i(rows), _i(cols), _i(per_thread), _i(row_groups),
+        _i(slice_cols), _i(chunk), _i(1 if read_first else 0)))
     return y
 
 

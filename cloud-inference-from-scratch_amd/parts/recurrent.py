@@ -256,7 +256,7 @@ class StateSpace(Part):
             raise ValueError(f"{num_heads} heads of {value_dim} in {groups} groups, normed in {norm_groups} parts: no equal parts")
         if taps > ops.MAX_CONV_TAPS or not eps > 0:
             raise ValueError(f"up to {ops.MAX_CONV_TAPS} taps and a positive eps, got {taps}, {eps}")
-        ops.plan_memory_walk(state, value_dim, False, False)  # (refuses memories the walk has no room for)
+        ops.plan_memory_walk(state, value_dim, False)  # (refuses memories the walk has no room for)
         self.hidden_size, self.num_heads, self.value_dim, self.state = hidden_size, num_heads, value_dim, state
         self.groups, self.taps, self.norm_groups, self.eps = groups, taps, norm_groups, float(eps)
         self.inner = num_heads * value_dim
@@ -333,7 +333,7 @@ class TimeMixing(Part):
                 raise ValueError(f"{name} must be a positive integer, got {value!r}")
         if not eps > 0:
             raise ValueError("eps must be positive")
-        ops.plan_memory_walk(head_dim, head_dim, True, True)  # (refuses memories the walk has no room for)
+        ops.plan_memory_walk(head_dim, head_dim, True)  # (refuses memories the walk has no room for)
         self.hidden_size, self.num_heads, self.head_dim, self.eps = hidden_size, num_heads, head_dim, float(eps)
         self.decay_rank = decay_rank  # None: whatever the checkpoint holds
         self.channels = num_heads * head_dim

@@ -110,10 +110,11 @@ class ScoredAttention(Part):
 
     def expected_tensors(self, prefix: str) -> dict[str, TensorSpec]:
         h, g, d, v, width = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, self.hidden_size
-        out = {prefix + "q": TensorSpec((h * d, width)), prefix + "o": TensorSpec((width, h * v))}
+        out = {prefix + "q": TensorSpec((h * d, width))}
         if self.own_kv:
             out[prefix + "k"] = TensorSpec((g * d, width))
             out[prefix + "v"] = TensorSpec((g * v, width))
+        out[prefix + "o"] = TensorSpec((width, h * v))
         if self.qkv_bias:
             out[prefix + "q.b"] = TensorSpec((h * d,))
             if self.own_kv:

@@ -810,7 +810,7 @@ def register_routed_toy():
                                max_position=self.max_position_embeddings, factor=self.FACTOR)
             windowed = PartSpec.of("attention", **{**dict(plain_layer.mixer.params), "window": self.WINDOW})
             slowed = PartSpec.of("attention", **{**dict(plain_layer.mixer.params), "position": slow})
-            routed = PartSpec.of("routed_experts", hidden_size=self.hidden_size, expert_size=self.EXPERT_SIZE,
+            routed = PartSpec.of("toy_routed_experts", hidden_size=self.hidden_size, expert_size=self.EXPERT_SIZE,
                                  experts=self.EXPERTS)
             first = LayerSpec(mixer=windowed, feed_forward=routed, norm1=plain_layer.norm1, norm2=plain_layer.norm2,
                               names=(("norm1", "input_layernorm"), ("mixer", "self_attn"),
@@ -822,7 +822,7 @@ def register_routed_toy():
                 layers=(first, second), order=(LayerCall(0, 0), LayerCall(1, 1)),
                 final_norm=base.final_norm, tie_word_embeddings=True, max_position=self.max_position_embeddings)
 
-    register_part("feed_forward", "routed_experts", RoutedExperts)
+    register_part("feed_forward", "toy_routed_experts", RoutedExperts)  # (a name of its own: the package has a part called routed_experts)
     register_part("position", "slow_rotary", SlowRotary)
     register_architecture("ToyRoutedWindowForCausalLM", RoutedToyConfig)
     return RoutedToyConfig

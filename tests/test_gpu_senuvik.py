@@ -25,7 +25,6 @@ pytestmark = pytest.mark.gpu
 # bfloat16: activations rounded to 8 bits between kernels, with these bold weights a few per cent at the worst row.
 LIMIT = {"float32": 2e-5, "bfloat16": 8e-2}
 RMS_LIMIT = {"float32": 1e-5, "bfloat16": 3e-2}
-DEEP_LIMIT = {"float32": 2e-5, "bfloat16": 2e-1}   # the worst row of models of up to six layers
 
 
 def plain_all(raw, weights, requests):
@@ -289,9 +288,15 @@ def test_random_configurations_and_traces(seed):
         rows = replay_util.by_position(steps, replay_util.drive_runner(runner, steps))
         assert rows
         worst, rms = su.spread(rows, plain)
-        # (up to six layers whose branches are all brought to the same size before they are added: bfloat16 rounding
-        # grows with the depth, evenly over the layers, and the worst row lies a few times above the rest)
-        assert worst <= DEEP_LIMIT[dtype] and rms <= RMS_LIMIT[dtype], (dtype, worst, rms, raw)
+        if dtype == "float32":
+            assert worst <= LIMIT[dtype] and rms <= RMS_LIMIT[dtype], (dtype, worst, rms, raw)
+        else:
+            # up to six layers whose branches are all brought to the same size before they are added: what bfloat16
+            # costs grows with the depth, evenly over the layers, and differs from model to model.  It is measured,
+            # not assumed: the engine has to be closer to the float32 logits than the plain implementation run in
+            # bfloat16 throughout is.
+            rough = {rid: ps.forward(raw, weights, tokens, dtype=torch.bfloat16) for rid, tokens in requests.items()}
+            replay_util.closer_than_plain_bfloat16(rows, plain, rough)
         assert runner.cache.stats().slots_used == 0 and runner.cache.stats().pages_used == 0
 
 
