@@ -229,7 +229,8 @@ shift_mix_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ be
     const T* row = h + static_cast<size_t>(token) * ldh;
     const T* prev = h + static_cast<size_t>(token - 1) * ldh;
     const float* kept = before + static_cast<size_t>(seq_slot[seq]) * width;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    // (blockIdx.y: the token's channels in blocks, so that a single token's row is not one thread's loop of loads)
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += blockDim.x * gridDim.y) {
         const float x = to_float(row[c]);
         const float d = (first ? kept[c] : to_float(prev[c])) - x;
         for (int s = 0; s < n_mix; ++s)
@@ -239,11 +240,12 @@ shift_mix_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ be
 }
 
 // w[t, c] = exp(-exp(w2[c, :] . tanh(low[t, :]) + w0[c])): the decay of every key channel from the low-rank
-// projection of its mix (float32 [tokens, rank]).  One workgroup per token; tanh(low) is staged in LDS.  Also moves
-// the token-shift state on: the step's last token of every sequence leaves its input row there.
+// projection of its mix (float32 [tokens, rank]).  `w2t` is w2 transposed, [rank, channels], so that neighbouring
+// threads read neighbouring numbers.  A workgroup per (token, block of channels); tanh(low) is staged in LDS.  Also
+// moves the token-shift state on: the step's last token of every sequence leaves its input row there.
 template <typename T>
 __global__ void __launch_bounds__(256)
-time_decay_kernel(const float* __restrict__ low, const T* __restrict__ w2, const float* __restrict__ w0,
+time_decay_kernel(const float* __restrict__ low, const T* __restrict__ w2t, const float* __restrict__ w0,
                   float* __restrict__ decay, int channels, int rank, const T* __restrict__ h, long ldh,
                   float* __restrict__ before, const int* __restrict__ seq_of_token, const int* __restrict__ seq_slot,
                   const int* __restrict__ q_start_loc, int width) {
@@ -251,17 +253,21 @@ time_decay_kernel(const float* __restrict__ low, const T* __restrict__ w2, const
     const int token = blockIdx.x;
     for (int r = threadIdx.x; r < rank; r += blockDim.x) bent[r] = tanhf(low[static_cast<size_t>(token) * rank + r]);
     __syncthreads();
-    for (int c = threadIdx.x; c < channels; c += blockDim.x) {
-        const T* row = w2 + static_cast<size_t>(c) * rank;
-        float sum = 0.f;
-        for (int r = 0; r < rank; ++r) sum = fmaf(to_float(row[r]), bent[r], sum);
-        decay[static_cast<size_t>(token) * channels + c] = expf(-expf(sum + w0[c]));
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < channels; c += blockDim.x * gridDim.y) {
+        float sum = 0.f, sum1 = 0.f;
+        int r = 0;
+        for (; r + 1 < rank; r += 2) {
+            sum = fmaf(to_float(w2t[static_cast<size_t>(r) * channels + c]), bent[r], sum);
+            sum1 = fmaf(to_float(w2t[static_cast<size_t>(r + 1) * channels + c]), bent[r + 1], sum1);
+        }
+        if (r < rank) sum = fmaf(to_float(w2t[static_cast<size_t>(r) * channels + c]), bent[r], sum);
+        decay[static_cast<size_t>(token) * channels + c] = expf(-expf((sum + sum1) + w0[c]));
     }
     const int seq = seq_of_token[token];
     if (token + 1 == q_start_loc[seq + 1]) {
         float* kept = before + static_cast<size_t>(seq_slot[seq]) * width;
         const T* row = h + static_cast<size_t>(token) * ldh;
-        for (int c = threadIdx.x; c < width; c += blockDim.x) kept[c] = to_float(row[c]);
+        for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += blockDim.x * gridDim.y) kept[c] = to_float(row[c]);
     }
 }
 
@@ -375,32 +381,37 @@ CIE_API int cie_shift_mix(void* stream, int dtype, const void* h, long ldh, cons
     if (tokens < 0 || width <= 0 || n_mix <= 0 || ldh < width || !before || !mu) return CIE_BAD_ARGUMENT;
     if (tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int blocks = (width + 255) / 256;
+    const dim3 grid(tokens, tokens >= 512 ? 1 : (blocks < 32 ? blocks : 32));
     if (dtype == CIE_F32)
-        shift_mix_kernel<float><<<tokens, 256, 0, s>>>(static_cast<const float*>(h), ldh, before, mu, seq_of_token, seq_slot,
+        shift_mix_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(h), ldh, before, mu, seq_of_token, seq_slot,
                                                       q_start_loc, static_cast<float*>(mixes), tokens, width, n_mix);
     else if (dtype == CIE_BF16)
-        shift_mix_kernel<bf16_t><<<tokens, 256, 0, s>>>(static_cast<const bf16_t*>(h), ldh, before, mu, seq_of_token, seq_slot,
+        shift_mix_kernel<bf16_t><<<grid, 256, 0, s>>>(static_cast<const bf16_t*>(h), ldh, before, mu, seq_of_token, seq_slot,
                                                        q_start_loc, static_cast<bf16_t*>(mixes), tokens, width, n_mix);
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();
 }
 
-CIE_API int cie_time_decay(void* stream, int dtype, const float* low, const void* w2, const float* w0, float* decay,
+CIE_API int cie_time_decay(void* stream, int dtype, const float* low, const void* w2t, const float* w0, float* decay,
                            int tokens, int channels, int rank, const void* h, long ldh, float* before,
                            const int* seq_of_token, const int* seq_slot, const int* q_start_loc, int width) {
-    if (tokens < 0 || channels <= 0 || rank <= 0 || rank > 8192 || width <= 0 || ldh < width || !low || !w2 || !w0 ||
+    if (tokens < 0 || channels <= 0 || rank <= 0 || rank > 8192 || width <= 0 || ldh < width || !low || !w2t || !w0 ||
         !decay || !h || !before)
         return CIE_BAD_ARGUMENT;
     if (tokens == 0) return CIE_OK;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t lds = static_cast<size_t>(rank) * sizeof(float);
+    const int most = channels > width ? channels : width;
+    const int blocks = (most + 255) / 256;
+    const dim3 grid(tokens, tokens >= 512 ? (blocks < 2 ? blocks : 2) : (blocks < 32 ? blocks : 32));
     if (dtype == CIE_F32)
-        time_decay_kernel<float><<<tokens, 256, lds, s>>>(low, static_cast<const float*>(w2), w0, decay, channels, rank,
+        time_decay_kernel<float><<<grid, 256, lds, s>>>(low, static_cast<const float*>(w2t), w0, decay, channels, rank,
                                                          static_cast<const float*>(h), ldh, before, seq_of_token,
                                                          seq_slot, q_start_loc, width);
     else if (dtype == CIE_BF16)
-        time_decay_kernel<bf16_t><<<tokens, 256, lds, s>>>(low, static_cast<const bf16_t*>(w2), w0, decay, channels, rank,
+        time_decay_kernel<bf16_t><<<grid, 256, lds, s>>>(low, static_cast<const bf16_t*>(w2t), w0, decay, channels, rank,
                                                           static_cast<const bf16_t*>(h), ldh, before, seq_of_token,
                                                           seq_slot, q_start_loc, width);
     else

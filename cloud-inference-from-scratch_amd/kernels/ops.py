@@ -1252,27 +1252,27 @@ def shift_mix(h: torch.Tensor, before: torch.Tensor, mu: torch.Tensor, seq_of_to
     return mixes
 
 
-def time_decay(low: torch.Tensor, w2: torch.Tensor, w0: torch.Tensor, h: torch.Tensor, before: torch.Tensor,
+def time_decay(low: torch.Tensor, w2t: torch.Tensor, w0: torch.Tensor, h: torch.Tensor, before: torch.Tensor,
                seq_of_token: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor) -> torch.Tensor:
-    """``exp(-exp(w2 tanh(low) + w0))``, float32 [T, C]: ``low`` float32 [T, rank], ``w2`` [C, rank] in h's type,
-    ``w0`` float32 [C].  Also leaves the last row of ``h`` of every sequence of the step in ``before`` (the token-shift
-    state that ``shift_mix`` reads at the next step)."""
+    """``exp(-exp(tanh(low) w2t + w0))``, float32 [T, C]: ``low`` float32 [T, rank], ``w2t`` [rank, C] in h's type
+    (the second small product's weight, transposed), ``w0`` float32 [C].  Also leaves the last row of ``h`` of every
+    sequence of the step in ``before`` (the token-shift state that ``shift_mix`` reads at the next step)."""
     _gpu("low", low, torch.float32, 2)
     tokens, rank = low.shape
     if not (h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _CODES and h.shape[0] == tokens):
         raise ValueError("h must be a float32 or bfloat16 GPU matrix with unit inner stride, a row per token")
-    _gpu("w2", w2, h.dtype, 2)
-    channels = w2.shape[0]
+    _gpu("w2t", w2t, h.dtype, 2)
+    channels = w2t.shape[1]
     _gpu("w0", w0, torch.float32, 1)
     _gpu("before", before, torch.float32, 2)
-    if w2.shape[1] != rank or w0.shape[0] != channels or before.shape[1] != h.shape[1]:
-        raise ValueError(f"w2 {tuple(w2.shape)}, w0 {tuple(w0.shape)}, before {tuple(before.shape)} do not fit")
+    if w2t.shape[0] != rank or w0.shape[0] != channels or before.shape[1] != h.shape[1]:
+        raise ValueError(f"w2t {tuple(w2t.shape)}, w0 {tuple(w0.shape)}, before {tuple(before.shape)} do not fit")
     for name, meta in (("seq_of_token", seq_of_token), ("seq_slot", seq_slot), ("q_start_loc", q_start_loc)):
         _gpu(name, meta, torch.int32, 1)
     decay = torch.empty((tokens, channels), dtype=torch.float32, device=low.device)
     ldh = h.stride(0) if tokens > 1 else max(h.stride(0), h.shape[1])
     _run("cie_time_decay", load_library().cie_time_decay(
-        _stream(), _i(_code(h.dtype)), _ptr(low), _ptr(w2), _ptr(w0), _ptr(decay), _i(tokens), _i(channels), _i(rank),
+        _stream(), _i(_code(h.dtype)), _ptr(low), _ptr(w2t), _ptr(w0), _ptr(decay), _i(tokens), _i(channels), _i(rank),
         _ptr(h), ldh, _ptr(before), _ptr(seq_of_token), _ptr(seq_slot), _ptr(q_start_loc), _i(h.shape[1])))
     return decay
 

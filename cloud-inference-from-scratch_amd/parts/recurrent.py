@@ -360,9 +360,10 @@ class TimeMixing(Part):
         self.mu = torch.stack([tensors[prefix + "mu." + name].float() for name in self.MIXES]).contiguous()
         self.w_r, self.w_k, self.w_v, self.w_g = (tensors[prefix + name].contiguous() for name in ("r", "k", "v", "g"))
         self.w_1 = tensors[prefix + "w1"].contiguous()
-        self.w_2 = tensors[prefix + "w2"].contiguous()
-        if self.w_1.shape[0] != self.w_2.shape[1]:
-            raise ValueError(f"{prefix}w1 {tuple(self.w_1.shape)} and {prefix}w2 {tuple(self.w_2.shape)} disagree on the rank")
+        w_2 = tensors[prefix + "w2"]
+        if self.w_1.shape[0] != w_2.shape[1]:
+            raise ValueError(f"{prefix}w1 {tuple(self.w_1.shape)} and {prefix}w2 {tuple(w_2.shape)} disagree on the rank")
+        self.w_2t = w_2.t().contiguous()  # [rank, channels]: the decay kernel's threads read neighbouring channels
         self.w_0 = tensors[prefix + "w0"].float().contiguous()
         self.bonus = tensors[prefix + "u"].float().contiguous()
         self.norm_weight = tensors[prefix + "norm"].float().contiguous()
@@ -385,7 +386,7 @@ class TimeMixing(Part):
         v = linear(mixes[2], self.w_v, out_dtype=f32)
         gate = linear(mixes[3], self.w_g)
         low = linear(mixes[4], self.w_1, out_dtype=f32)
-        decay = ops.time_decay(low, self.w_2, self.w_0, x, before, batch.seq_of_token, batch.seq_slot, batch.q_start_loc)
+        decay = ops.time_decay(low, self.w_2t, self.w_0, x, before, batch.seq_of_token, batch.seq_slot, batch.q_start_loc)
         y = ops.memory_walk(decay, k, r, v, memory, batch.seq_slot, batch.q_start_loc, batch.sequences, self.num_heads,
                             self.head_dim, self.head_dim, bonus=self.bonus, read_first=True)
         out = ops.gated_group_norm(y, gate, self.norm_weight, self.num_heads, self.eps, x.dtype, gate_first=False)

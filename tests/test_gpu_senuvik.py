@@ -714,7 +714,7 @@ def test_token_shift_decays_and_the_convolution_carry_their_state():
     assert torch.allclose(mixes.cpu(), want, atol=1e-6)
     low = torch.randn(tokens, rank, generator=g)
     w2, w0 = torch.randn(channels, rank, generator=g), torch.randn(channels, generator=g)
-    decay = ops.time_decay(low.cuda(), w2.cuda(), w0.cuda(), h.cuda(), state, seq_of_token, slot_t, q_start_loc)
+    decay = ops.time_decay(low.cuda(), w2.t().contiguous().cuda(), w0.cuda(), h.cuda(), state, seq_of_token, slot_t, q_start_loc)
     assert torch.allclose(decay.cpu(), torch.exp(-torch.exp(torch.tanh(low) @ w2.t() + w0)), atol=1e-6, rtol=1e-5)
     kept = before.clone()
     first = 0
