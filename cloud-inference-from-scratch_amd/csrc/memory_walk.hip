@@ -199,19 +199,289 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------- the walk in blocks
+// The first form of the walk (one decay per head and token, the read-out behind the update) for sequences that
+// bring many tokens: blocks of 32 tokens on the matrix cores, float32 throughout (`v_mfma_f32_16x16x4_f32`), and only
+// what has to wait for the block before it waits.  With S the memory in front of a block of n tokens, i and j tokens
+// of the block, L_i the sum of the logarithms of the decays of the block's tokens 0 .. i, and w_j = val_j * scale_j:
+//     y_i   = exp(L_i) * (S^T out_i)  +  sum_{j <= i} exp(L_i - L_j) (out_i . in_j) w_j   (+ skip * val_i)
+//     S_new = exp(L_(n-1)) * S  +  sum_j exp(L_(n-1) - L_j) in_j w_j^T
+// (every exponent is at most zero).  Three kernels, as for the memory with a fixed decay in recurrent.hip:
+// `walk_block_sums_kernel`, every block at once, makes the second term of y and of S_new (into the block's place of
+// `sums`) and the block's whole decay; `walk_scan_kernel`, one thread per number of the memory, goes over a
+// sequence's blocks in order: the block's place gets the S in front of it, and S moves on; `walk_block_reads_kernel`,
+// every block at once, adds the first term of y.  Block b of sequence s has place first_token(s) / 32 + s + b.  Rows
+// are padded to whole tiles of 16 (`padded`), a workgroup takes up to 128 columns (a panel) rounded up to tiles of
+// 16 (`cols16` columns a row of `sums`).  Operand layouts of the 16 x 16 x 4 product: lane (l16 = lane % 16,
+// g = lane / 16) gives A[l16][g] and B[g][l16] and gets rows 4 g .. 4 g + 3 of column l16; which four numbers of a
+// sum a product takes does not matter as long as both operands agree, so a lane reads four neighbouring numbers at
+// once and spends them on four products.
+typedef float acc4_t __attribute__((ext_vector_type(4)));
+constexpr int kBlockTokens = 32;
+constexpr int kPanelCols = 128;
+constexpr int kScoreStride = kBlockTokens + 4;
+
+// rows of a panel of values in LDS start 16 banks apart: the four tokens that a product reads then touch every bank
+__host__ __device__ inline int panel_stride(int cols) { return cols % 32 == 0 ? cols + 16 : cols; }
+
+struct BlockArgs {
+    const float* log_decay;  // log_decay[t * ld_decay + head]
+    long ld_decay;
+    const float* in;         // in[t * ld_in + (head / heads_per_group) * rows + n]
+    long ld_in;
+    const float* out;
+    long ld_out;
+    int heads_per_group;
+    const float* val;        // val[t * ld_val + head * cols + p]
+    long ld_val;
+    const float* val_scale;  // val_scale[t * ld_scale + head] or null
+    long ld_scale;
+    const float* skip;       // [heads] or null
+    float* state;            // [slots, heads, rows, cols]
+    const int* seq_slot;
+    const int* q_start_loc;
+    float* y;                // [tokens, heads * cols]
+    float* sums;             // [places, heads, padded, cols16]
+    float* totals;           // [places, heads]: exp of the block's summed log decays
+    int heads, rows, cols, padded, cols16;
+};
+
+// L_0 .. L_31 of a block into `cum` (tokens past the block's last repeat its L), by one thread
+__device__ __forceinline__ void block_logs(float* cum, const BlockArgs& a, int first_token, int cn, int head) {
+    if (threadIdx.x == 0) {
+        float sum = 0.f;
+        for (int t = 0; t < kBlockTokens; ++t) {
+            if (t < cn) sum += a.log_decay[static_cast<size_t>(first_token + t) * a.ld_decay + head];
+            cum[t] = sum;
+        }
+    }
+}
+
+// a block's rows of `src` (in or out) into LDS rows of `stride` floats; rows past the memory's last and tokens past
+// the block's last are zero
+__device__ __forceinline__ void stage_block_rows(float* dst, int stride, const float* __restrict__ src, long ld,
+                                                 int first_token, int cn, int offset, int rows, int padded) {
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    for (int t = wave; t < kBlockTokens; t += 4) {
+        const float* row = src + static_cast<size_t>(first_token + min(t, cn - 1)) * ld + offset;
+        for (int n = lane; n < padded; n += kWave) dst[t * stride + n] = (t < cn && n < rows) ? row[n] : 0.f;
+    }
+}
+
+__global__ void __launch_bounds__(256) walk_block_sums_kernel(BlockArgs a) {
+    const int seq = blockIdx.x / a.heads;
+    const int head = blockIdx.x - seq * a.heads;
+    const int first = a.q_start_loc[seq];
+    const int count = a.q_start_loc[seq + 1] - first;
+    const int c0 = blockIdx.y * kBlockTokens;
+    if (c0 >= count) return;                             // (the whole workgroup: the grid is sized for the longest sequence)
+    const int cn = min(kBlockTokens, count - c0);
+    const int panel0 = blockIdx.z * kPanelCols;
+    const int cols = min(kPanelCols, a.cols16 - panel0);
+    const int col_tiles = cols / 16;
+    const int padded = a.padded;
+    const int stride = padded + 4;
+    const int vstride = panel_stride(cols);
+    extern __shared__ float4 lds4[];
+    float* q_s = reinterpret_cast<float*>(lds4);          // [32][stride]: the read-out's rows
+    float* k_s = q_s + kBlockTokens * stride;            // [32][stride]: the update's rows
+    float* v_s = k_s + kBlockTokens * stride;            // [32][vstride]: the scaled values
+    float* p_s = v_s + kBlockTokens * vstride;           // [32][36]: exp(L_i - L_j) (out_i . in_j), zero above the diagonal
+    float* cum = p_s + kBlockTokens * kScoreStride;      // [32]
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int l16 = lane % 16;
+    const int g = lane / 16;
+    const int tiles = padded / 16;
+    const int offset = (head / a.heads_per_group) * a.rows;
+    block_logs(cum, a, first + c0, cn, head);
+    stage_block_rows(q_s, stride, a.out, a.ld_out, first + c0, cn, offset, a.rows, padded);
+    stage_block_rows(k_s, stride, a.in, a.ld_in, first + c0, cn, offset, a.rows, padded);
+    for (int t = wave; t < kBlockTokens; t += 4) {
+        const size_t token = static_cast<size_t>(first + c0 + min(t, cn - 1));
+        const float scale = a.val_scale ? a.val_scale[token * a.ld_scale + head] : 1.f;
+        const float* src = a.val + token * a.ld_val + head * a.cols;
+        for (int c = lane; c < cols; c += kWave)
+            v_s[t * vstride + c] = (t < cn && panel0 + c < a.cols) ? src[panel0 + c] * scale : 0.f;
+    }
+    __syncthreads();
+    {   // this wave's tile of the scores (the tile above the diagonal is zero)
+        const int ti = wave >> 1, tj = wave & 1;
+        acc4_t p = {0.f, 0.f, 0.f, 0.f};
+        if (tj <= ti) {
+            const float* qa = q_s + (16 * ti + l16) * stride + 4 * g;
+            const float* kb = k_s + (16 * tj + l16) * stride + 4 * g;
+            acc4_t p1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+            for (int m = 0; m < tiles; ++m) {
+                const float4 x = *reinterpret_cast<const float4*>(qa + 16 * m);
+                const float4 b = *reinterpret_cast<const float4*>(kb + 16 * m);
+                p = __builtin_amdgcn_mfma_f32_16x16x4f32(x.x, b.x, p, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(x.y, b.y, p1, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_f32_16x16x4f32(x.z, b.z, p, 0, 0, 0);
+                p1 = __builtin_amdgcn_mfma_f32_16x16x4f32(x.w, b.w, p1, 0, 0, 0);
+            }
+            p += p1;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i = 16 * ti + 4 * g + r, j = 16 * tj + l16;
+            p_s[i * kScoreStride + j] = i >= j ? p[r] * expf(cum[i] - cum[j]) : 0.f;
+        }
+    }
+    __syncthreads();
+    float k_fade[kBlockTokens / 4];
+#pragma unroll
+    for (int kk = 0; kk < kBlockTokens / 4; ++kk) k_fade[kk] = expf(cum[kBlockTokens - 1] - cum[4 * kk + g]);
+    const int place = first / kBlockTokens + seq + blockIdx.y;
+    if (threadIdx.x == 0 && blockIdx.z == 0) a.totals[static_cast<size_t>(place) * a.heads + head] = expf(cum[kBlockTokens - 1]);
+    float* sum_rows = a.sums + (static_cast<size_t>(place) * a.heads + head) * padded * a.cols16 + panel0;
+    const float skip = a.skip ? a.skip[head] : 0.f;
+    for (int ct = wave; ct < col_tiles; ct += 4) {       // this wave's tiles of columns
+        float vb[kBlockTokens / 4];
+#pragma unroll
+        for (int kk = 0; kk < kBlockTokens / 4; ++kk) vb[kk] = v_s[(4 * kk + g) * vstride + 16 * ct + l16];
+        // the block's own share of y
+        acc4_t o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < kBlockTokens / 4; ++kk) {
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[l16 * kScoreStride + 4 * kk + g], vb[kk], o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(p_s[(16 + l16) * kScoreStride + 4 * kk + g], vb[kk], o1, 0, 0, 0);
+        }
+        const int col = panel0 + 16 * ct + l16;
+        if (col < a.cols) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * g + r;
+                const size_t token = static_cast<size_t>(first + c0);
+                float* dst = a.y + token * a.heads * a.cols + head * a.cols + col;
+                const float* raw = a.val + token * a.ld_val + head * a.cols + col;
+                if (i < cn) dst[static_cast<size_t>(i) * a.heads * a.cols] = fmaf(skip, raw[static_cast<size_t>(i) * a.ld_val], o0[r]);
+                if (16 + i < cn)
+                    dst[static_cast<size_t>(16 + i) * a.heads * a.cols] = fmaf(skip, raw[static_cast<size_t>(16 + i) * a.ld_val], o1[r]);
+            }
+        }
+        // what the block adds to the memory
+        for (int rt = 0; rt < tiles; ++rt) {
+            acc4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < kBlockTokens / 4; ++kk)
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(k_s[(4 * kk + g) * stride + 16 * rt + l16] * k_fade[kk], vb[kk],
+                                                          acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum_rows[static_cast<size_t>(16 * rt + 4 * g + r) * a.cols16 + 16 * ct + l16] = acc[r];
+        }
+    }
+}
+
+// One thread per number of a head's memory (rows and columns padded as `sums` has them): over the sequence's blocks in
+// order, the block's place gets the memory in front of the block, and the memory moves on by the block's sum.
+__global__ void __launch_bounds__(256) walk_scan_kernel(BlockArgs a) {
+    const int seq = blockIdx.x / a.heads;
+    const int head = blockIdx.x - seq * a.heads;
+    const int e = blockIdx.y * blockDim.x + threadIdx.x;
+    if (e >= a.padded * a.cols16) return;
+    const int first = a.q_start_loc[seq];
+    const int count = a.q_start_loc[seq + 1] - first;
+    if (count <= 0) return;
+    const int row = e / a.cols16;
+    const int col = e - row * a.cols16;
+    const bool real = row < a.rows && col < a.cols;
+    float* mem = a.state + ((static_cast<size_t>(a.seq_slot[seq]) * a.heads + head) * a.rows + row) * a.cols + col;
+    float S = real ? *mem : 0.f;
+    const int blocks = (count + kBlockTokens - 1) / kBlockTokens;
+    const size_t place0 = static_cast<size_t>(first / kBlockTokens + seq);
+    const size_t step = static_cast<size_t>(a.heads) * a.padded * a.cols16;
+    float* at = a.sums + (place0 * a.heads + head) * a.padded * a.cols16 + e;
+    const float* fade = a.totals + place0 * a.heads + head;
+    float add = at[0];
+    float whole = fade[0];
+    for (int b = 0; b < blocks; ++b) {
+        const int ahead = min(b + 1, blocks - 1);
+        const float next = at[static_cast<size_t>(ahead) * step];  // (asked for before this block's place is written)
+        const float next_whole = fade[static_cast<size_t>(ahead) * a.heads];
+        at[static_cast<size_t>(b) * step] = S;
+        S = fmaf(whole, S, add);
+        add = next;
+        whole = next_whole;
+    }
+    if (real) *mem = S;
+}
+
+__global__ void __launch_bounds__(256) walk_block_reads_kernel(BlockArgs a) {
+    const int seq = blockIdx.x / a.heads;
+    const int head = blockIdx.x - seq * a.heads;
+    const int first = a.q_start_loc[seq];
+    const int count = a.q_start_loc[seq + 1] - first;
+    const int c0 = blockIdx.y * kBlockTokens;
+    if (c0 >= count) return;
+    const int cn = min(kBlockTokens, count - c0);
+    const int panel0 = blockIdx.z * kPanelCols;
+    const int col_tiles = min(kPanelCols, a.cols16 - panel0) / 16;
+    const int padded = a.padded;
+    const int stride = padded + 4;
+    extern __shared__ float4 lds4[];
+    float* q_s = reinterpret_cast<float*>(lds4);          // [32][stride]
+    float* cum = q_s + kBlockTokens * stride;            // [32]
+    const int lane = threadIdx.x % kWave;
+    const int wave = threadIdx.x / kWave;
+    const int l16 = lane % 16;
+    const int g = lane / 16;
+    const int tiles = padded / 16;
+    block_logs(cum, a, first + c0, cn, head);
+    stage_block_rows(q_s, stride, a.out, a.ld_out, first + c0, cn, (head / a.heads_per_group) * a.rows, a.rows, padded);
+    __syncthreads();
+    const int place = first / kBlockTokens + seq + blockIdx.y;
+    const float* before = a.sums + (static_cast<size_t>(place) * a.heads + head) * padded * a.cols16 + panel0;
+    for (int ct = wave; ct < col_tiles; ct += 4) {
+        acc4_t o0 = {0.f, 0.f, 0.f, 0.f}, o1 = {0.f, 0.f, 0.f, 0.f};
+        const float* rows = before + static_cast<size_t>(4 * g) * a.cols16 + 16 * ct + l16;
+#pragma unroll 2
+        for (int m = 0; m < tiles; ++m) {
+            const float4 a0 = *reinterpret_cast<const float4*>(q_s + l16 * stride + 16 * m + 4 * g);
+            const float4 a1 = *reinterpret_cast<const float4*>(q_s + (16 + l16) * stride + 16 * m + 4 * g);
+            const float* s = rows + static_cast<size_t>(16 * m) * a.cols16;
+            const float b0 = s[0], b1 = s[a.cols16], b2 = s[2 * a.cols16], b3 = s[3 * a.cols16];
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.x, b0, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.x, b0, o1, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.y, b1, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.y, b1, o1, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.z, b2, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.z, b2, o1, 0, 0, 0);
+            o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a0.w, b3, o0, 0, 0, 0);
+            o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a1.w, b3, o1, 0, 0, 0);
+        }
+        const int col = panel0 + 16 * ct + l16;
+        if (col < a.cols) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * g + r;
+                float* dst = a.y + static_cast<size_t>(first + c0) * a.heads * a.cols + head * a.cols + col;
+                if (i < cn) dst[static_cast<size_t>(i) * a.heads * a.cols] += o0[r] * expf(cum[i]);
+                if (16 + i < cn) dst[static_cast<size_t>(16 + i) * a.heads * a.cols] += o1[r] * expf(cum[16 + i]);
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------- state-space steps
-// Per (token, head): the step size dt = softplus(raw + bias) and the decay exp(-exp(a_log) * dt), float32.
+// Per (token, head): the step size dt = softplus(raw + bias), the decay's logarithm -exp(a_log) * dt and the decay,
+// float32.
 template <typename T>
 __global__ void __launch_bounds__(256)
 space_steps_kernel(const T* __restrict__ raw, long ld, const float* __restrict__ bias, const float* __restrict__ a_log,
-                   float* __restrict__ steps, float* __restrict__ decay, long count, int heads) {
+                   float* __restrict__ steps, float* __restrict__ decay, float* __restrict__ log_decay, long count,
+                   int heads) {
     const long idx = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= count) return;
     const long token = idx / heads;
     const int head = static_cast<int>(idx - token * heads);
     const float dt = softplus_f(to_float(raw[token * ld + head]) + bias[head]);
+    const float fade = -expf(a_log[head]) * dt;
     steps[idx] = dt;
-    decay[idx] = expf(-expf(a_log[head]) * dt);
+    log_decay[idx] = fade;
+    decay[idx] = expf(fade);
 }
 
 // ---------------------------------------------------------------------------------------------- token shift
@@ -359,17 +629,52 @@ CIE_API int cie_memory_walk(void* stream, const float* decay, long ld_decay, con
     return cie_after_launch();
 }
 
+// The first form of the walk in blocks of 32 tokens on the matrix cores (see above).  `sums` holds
+// (tokens / 32 + sequences + 1) * heads * padded * cols16 floats and `totals` (tokens / 32 + sequences + 1) * heads,
+// with padded and cols16 the rows and columns rounded up to multiples of 16.
+CIE_API int cie_memory_walk_blocks(void* stream, const float* log_decay, long ld_decay, const float* in, long ld_in,
+                                   const float* out, long ld_out, int heads_per_group, const float* val, long ld_val,
+                                   const float* val_scale, long ld_scale, const float* skip, float* state,
+                                   const int* seq_slot, const int* q_start_loc, float* y, float* sums, float* totals,
+                                   int tokens, int sequences, int heads, int rows, int cols) {
+    if (sequences < 0 || tokens < 0 || heads <= 0 || rows <= 0 || cols <= 0 || heads_per_group <= 0 ||
+        heads % heads_per_group || !log_decay || !in || !out || !val || !state || !y || !sums || !totals)
+        return CIE_BAD_ARGUMENT;
+    const int padded = (rows + 15) / 16 * 16;
+    const int cols16 = (cols + 15) / 16 * 16;
+    const int panels = (cols16 + kPanelCols - 1) / kPanelCols;
+    const int most_blocks = (tokens + kBlockTokens - 1) / kBlockTokens;  // (of one sequence: the grid's second size)
+    const size_t sums_lds = sizeof(float) * (2 * static_cast<size_t>(kBlockTokens) * (padded + 4) +
+                                             kBlockTokens * panel_stride(cols16 < kPanelCols ? cols16 : kPanelCols) +
+                                             kBlockTokens * kScoreStride + kBlockTokens + 4);
+    const size_t reads_lds = sizeof(float) * (static_cast<size_t>(kBlockTokens) * (padded + 4) + kBlockTokens + 4);
+    if (sums_lds > 64 * 1024 || most_blocks > 65535 || panels > 65535 || static_cast<long>(sequences) * heads > 0x7fffffffL)
+        return CIE_BAD_ARGUMENT;
+    if (sequences == 0 || tokens == 0) return CIE_OK;
+    BlockArgs a{log_decay, ld_decay, in, ld_in, out, ld_out, heads_per_group, val, ld_val, val_scale, ld_scale, skip,
+                state, seq_slot, q_start_loc, y, sums, totals, heads, rows, cols, padded, cols16};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 block_grid(sequences * heads, most_blocks, panels);
+    walk_block_sums_kernel<<<block_grid, 256, sums_lds, s>>>(a);
+    if (hipGetLastError() != hipSuccess) return CIE_LAUNCH_FAILED;
+    const dim3 scan_grid(sequences * heads, (padded * cols16 + 255) / 256);
+    walk_scan_kernel<<<scan_grid, 256, 0, s>>>(a);
+    if (hipGetLastError() != hipSuccess) return CIE_LAUNCH_FAILED;
+    walk_block_reads_kernel<<<block_grid, 256, reads_lds, s>>>(a);
+    return cie_after_launch();
+}
+
 CIE_API int cie_space_steps(void* stream, int dtype, const void* raw, long ld, const float* bias, const float* a_log,
-                            float* steps, float* decay, int tokens, int heads) {
-    if (tokens < 0 || heads <= 0 || ld < heads || !bias || !a_log || !steps || !decay) return CIE_BAD_ARGUMENT;
+                            float* steps, float* decay, float* log_decay, int tokens, int heads) {
+    if (tokens < 0 || heads <= 0 || ld < heads || !bias || !a_log || !steps || !decay || !log_decay) return CIE_BAD_ARGUMENT;
     if (tokens == 0) return CIE_OK;
     const long count = static_cast<long>(tokens) * heads;
     const unsigned blocks = static_cast<unsigned>((count + 255) / 256);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == CIE_F32)
-        space_steps_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(raw), ld, bias, a_log, steps, decay, count, heads);
+        space_steps_kernel<float><<<blocks, 256, 0, s>>>(static_cast<const float*>(raw), ld, bias, a_log, steps, decay, log_decay, count, heads);
     else if (dtype == CIE_BF16)
-        space_steps_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(raw), ld, bias, a_log, steps, decay, count, heads);
+        space_steps_kernel<bf16_t><<<blocks, 256, 0, s>>>(static_cast<const bf16_t*>(raw), ld, bias, a_log, steps, decay, log_decay, count, heads);
     else
         return CIE_BAD_ARGUMENT;
     return cie_after_launch();

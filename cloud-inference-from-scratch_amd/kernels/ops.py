@@ -1134,6 +1134,8 @@ def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, g
 WALK_ROWS = (4, 8, 16, 32, 64)   # rows of a memory that one thread of the walk keeps in registers
 WALK_MAX_ROWS = 1024
 WALK_LDS_BYTES = 48 * 1024
+WALK_BLOCKS_FROM = 16            # tokens a sequence (on average) from which the first form of the walk goes in blocks
+WALK_BLOCKS_MAX_BYTES = 2 << 30  # ... while the blocks' sums fit this much scratch memory
 
 
 def plan_memory_walk(rows: int, cols: int, time_form: bool, units: int = 1) -> tuple[int, int, int, int]:
@@ -1161,14 +1163,17 @@ def memory_walk(decay: torch.Tensor, in_rows: torch.Tensor, out_rows: torch.Tens
                 state: torch.Tensor, seq_slot: torch.Tensor, q_start_loc: torch.Tensor, sequences: int, heads: int,
                 rows: int, cols: int, heads_per_group: int = 1, bonus: Optional[torch.Tensor] = None,
                 value_scale: Optional[torch.Tensor] = None, skip: Optional[torch.Tensor] = None,
-                read_first: bool = False) -> torch.Tensor:
+                read_first: bool = False, log_decay: Optional[torch.Tensor] = None,
+                blocks: Optional[bool] = None) -> torch.Tensor:
     """The walk of ``csrc/memory_walk.hip`` over a step's tokens: per head a float32 memory ``S`` [rows, cols] in
     ``state`` [slots, heads, rows, cols], ``S <- decay * S + in (x) (value * value_scale)`` token by token, and the
     read-out ``y = S^T out + skip * value`` behind the update, or (``read_first``) ``y = (S + (bonus * in) (x) value)^T
     out`` in front of it.  All operands float32 views with unit inner stride: ``decay`` [T, heads] (one per head and
     token) or [T, heads * rows]; ``in_rows``, ``out_rows`` [T, (heads / heads_per_group) * rows]; ``values``
     [T, heads * cols]; ``bonus`` [heads, rows]; ``value_scale`` [T, heads]; ``skip`` [heads].  Returns y, float32
-    [T, heads * cols]."""
+    [T, heads * cols].  With ``log_decay`` (float32 [T, heads], the decays' logarithms; the first form only) sequences
+    that bring ``WALK_BLOCKS_FROM`` tokens and more on average are walked in blocks of 32 tokens on the matrix cores
+    (``blocks``: force it or forbid it); the sums come in another order, a difference of float32 rounding."""
     tokens = values.shape[0]
     groups_of_heads = heads // heads_per_group
     if heads % heads_per_group:
@@ -1202,6 +1207,26 @@ def memory_walk(decay: torch.Tensor, in_rows: torch.Tensor, out_rows: torch.Tens
     per_thread, row_groups, slice_cols, chunk = plan_memory_walk(rows, cols, per_row, sequences * heads)
     y = torch.empty((tokens, heads * cols), dtype=torch.float32, device=values.device)
     ld = lambda t: t.stride(0) if tokens > 1 else max(t.stride(0), t.shape[1])
+    if blocks is None:
+        blocks = tokens >= WALK_BLOCKS_FROM * max(sequences, 1)
+    if blocks and log_decay is not None and not read_first and bonus is None and sequences > 0:
+        padded, cols16 = -(-rows // 16) * 16, -(-cols // 16) * 16
+        panel = min(cols16, 128)
+        lds = 4 * (2 * 32 * (padded + 4) + 32 * (panel + 16 if panel % 32 == 0 else panel) + 32 * 36 + 36)
+        places = tokens // 32 + sequences + 1
+        scratch = places * heads * padded * cols16 * 4
+        if lds <= 64 * 1024 and scratch <= WALK_BLOCKS_MAX_BYTES and tokens <= 32 * 65535:
+            if not (log_decay.is_cuda and log_decay.dtype == torch.float32 and tuple(log_decay.shape) == (tokens, heads)
+                    and log_decay.stride(1) == 1):
+                raise ValueError(f"log_decay must be float32 [{tokens}, {heads}]")
+            sums = torch.empty(places * heads * padded * cols16, dtype=torch.float32, device=values.device)
+            totals = torch.empty(places * heads, dtype=torch.float32, device=values.device)
+            _run("cie_memory_walk_blocks", load_library().cie_memory_walk_blocks(
+                _stream(), _ptr(log_decay), ld(log_decay), _ptr(in_rows), ld(in_rows), _ptr(out_rows), ld(out_rows),
+                _i(heads_per_group), _ptr(values), ld(values), _ptr(value_scale), ld_scale, _ptr(skip), _ptr(state),
+                _ptr(seq_slot), _ptr(q_start_loc), _ptr(y), _ptr(sums), _ptr(totals), _i(tokens), _i(sequences), _i(heads),
+                _i(rows), _i(cols)))
+            return y
     _run("cie_memory_walk", load_library().cie_memory_walk(
         _stream(), _ptr(decay), ld(decay), _ptr(in_rows), ld(in_rows), _ptr(out_rows), ld(out_rows), _i(heads_per_group),
         _ptr(bonus), _ptr(values), ld(values), _ptr(value_scale), ld_scale, _ptr(skip), _ptr(state), _ptr(seq_slot),
@@ -1210,9 +1235,10 @@ def memory_walk(decay: torch.Tensor, in_rows: torch.Tensor, out_rows: torch.Tens
     return y
 
 
-def space_steps(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
-    """Step sizes and decays of a state-space layer: ``dt = softplus(raw + bias)`` and ``exp(-exp(a_log) * dt)`` per
-    token and head, both float32 [T, heads].  ``raw`` [T, heads] (a view with unit inner stride); bias, a_log float32."""
+def space_steps(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Step sizes and decays of a state-space layer: ``dt = softplus(raw + bias)``, ``exp(-exp(a_log) * dt)`` and the
+    decay's logarithm ``-exp(a_log) * dt`` per token and head, all float32 [T, heads].  ``raw`` [T, heads] (a view
+    with unit inner stride); bias, a_log float32."""
     if not (raw.is_cuda and raw.dim() == 2 and raw.stride(1) == 1 and raw.dtype in _CODES):
         raise ValueError("raw must be a float32 or bfloat16 GPU matrix with unit inner stride")
     tokens, heads = raw.shape
@@ -1220,12 +1246,12 @@ def space_steps(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor) -> t
         _gpu(name, t, torch.float32, 1)
         if t.shape[0] != heads:
             raise ValueError(f"{name} must be [{heads}]")
-    steps = torch.empty((tokens, heads), dtype=torch.float32, device=raw.device)
-    decay = torch.empty((tokens, heads), dtype=torch.float32, device=raw.device)
+    made = torch.empty((3, tokens, heads), dtype=torch.float32, device=raw.device)
     ld = raw.stride(0) if tokens > 1 else max(raw.stride(0), heads)
     _run("cie_space_steps", load_library().cie_space_steps(_stream(), _i(_code(raw.dtype)), _ptr(raw), ld, _ptr(bias),
-                                                           _ptr(a_log), _ptr(steps), _ptr(decay), _i(tokens), _i(heads)))
-    return steps, decay
+                                                           _ptr(a_log), _ptr(made[0]), _ptr(made[1]), _ptr(made[2]),
+                                                           _i(tokens), _i(heads)))
+    return made[0], made[1], made[2]
 
 
 def shift_mix(h: torch.Tensor, before: torch.Tensor, mu: torch.Tensor, seq_of_token: torch.Tensor,

@@ -308,11 +308,13 @@ class StateSpace(Part):
         mixed = ops.causal_conv(taken, self.conv_w, self.conv_b, past, batch.seq_of_token, batch.seq_slot,
                                 batch.q_start_loc, activation="silu", out_dtype=torch.float32)
         ops.conv_keep(taken, past, batch.seq_slot, batch.q_start_loc, batch.sequences, self.taps)
-        steps, decay = ops.space_steps(raw_dt, self.dt_bias, self.a_log)
+        steps, decay, log_decay = ops.space_steps(raw_dt, self.dt_bias, self.a_log)
+        # (prompts' portions walk in blocks on the matrix cores, single tokens and short portions token by token:
+        # which of the two follows from the step's shape, which a captured step repeats)
         y = ops.memory_walk(decay, mixed[:, inner: inner + bc], mixed[:, inner + bc:], mixed[:, :inner], memory,
                             batch.seq_slot, batch.q_start_loc, batch.sequences, self.num_heads, self.state,
                             self.value_dim, heads_per_group=self.num_heads // self.groups, value_scale=steps,
-                            skip=self.skip)
+                            skip=self.skip, log_decay=log_decay)
         out = ops.gated_group_norm(y, z, self.norm_weight, self.norm_groups, self.eps, x.dtype, gate_first=True)
         return linear(out, self.w_o)
 

@@ -559,7 +559,7 @@ def test_the_memory_walk_against_a_loop(shape):
 
     heads, rows, cols, per_group, time_form = shape
     g = torch.Generator().manual_seed(rows * 7 + cols)
-    lengths = [1, 37, 2, 19]
+    lengths = [1, 37, 2, 19] if rows < 200 else [1, 70, 2, 33]
     slots = [3, 0, 4, 1]
     tokens = sum(lengths)
     q_start_loc, _ = _meta(lengths)
@@ -605,6 +605,16 @@ def test_the_memory_walk_against_a_loop(shape):
     assert torch.allclose(state_gpu.double().cpu(), want_state, rtol=1e-4, atol=1e-4)
     untouched = [s for s in range(6) if s not in slots]
     assert torch.equal(state_gpu[untouched].cpu(), state[untouched])
+    if not time_form:
+        # the same in blocks of 32 tokens on the matrix cores (sequences of 1, 37, 2 and 19 tokens: whole blocks, rests)
+        state_gpu = state.cuda()
+        got = ops.memory_walk(cuda(decay), wide[:, :n], wide[:, n:2 * n], wide[:, 2 * n:], state_gpu,
+                              torch.tensor(slots, dtype=torch.int32, device="cuda"), q_start_loc, len(lengths), heads, rows,
+                              cols, heads_per_group=per_group, value_scale=cuda(scale), skip=cuda(skip),
+                              log_decay=torch.log(decay).cuda(), blocks=True)
+        assert torch.allclose(got.double().cpu(), want, rtol=1e-4, atol=1e-4)
+        assert torch.allclose(state_gpu.double().cpu(), want_state, rtol=1e-4, atol=1e-4)
+        assert torch.equal(state_gpu[untouched].cpu(), state[untouched])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
