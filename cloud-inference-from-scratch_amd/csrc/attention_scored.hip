@@ -32,6 +32,44 @@ using namespace cie_attention;
 namespace {
 
 // ------------------------------------------------------------------------------------------------ prepare
+// A wave's sum of the squares of n numbers: sixteen bytes a lane and load where the numbers start at a multiple of
+// sixteen bytes (every wave of a token sums the whole projection again under the norm over all heads: the loads
+// are what that costs).
+__device__ __forceinline__ float wave_sum_squares(const float* p, int n, int lane) {
+    float sum = 0.f;
+    int done = 0;
+    if ((reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+        for (int d = 4 * lane; d + 3 < n; d += 4 * kWave) {
+            const float4 v = *reinterpret_cast<const float4*>(p + d);
+            sum += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+        }
+        done = n & ~3;
+    }
+    for (int d = done + lane; d < n; d += kWave) sum += p[d] * p[d];
+    return wave_sum(sum);
+}
+__device__ __forceinline__ float wave_sum_squares(const bf16_t* p, int n, int lane) {
+    float sum = 0.f;
+    int done = 0;
+    if ((reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+        for (int d = 8 * lane; d + 7 < n; d += 8 * kWave) {
+            const uint4 raw = *reinterpret_cast<const uint4*>(p + d);
+            const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float lo = __uint_as_float(w[i] << 16), hi = __uint_as_float(w[i] & 0xffff0000u);
+                sum += lo * lo + hi * hi;
+            }
+        }
+        done = n & ~7;
+    }
+    for (int d = done + lane; d < n; d += kWave) {
+        const float x = to_float(p[d]);
+        sum += x * x;
+    }
+    return wave_sum(sum);
+}
+
 // One wave per (token, head slot): slots 0..H-1 queries, H..H+G-1 keys, H+G..H+2G-1 values.
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -74,12 +112,7 @@ heads_prepare_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int
     if (norm_mode == 3) {  // one root mean square over all heads of the projection; the weight has a number for each
         const int all = (is_q ? q_heads : kv_heads) * dim;
         const T* whole = row + (is_q ? q_off : k_off);
-        float sum_sq = 0.f;
-        for (int d = lane; d < all; d += kWave) {
-            const float x = to_float(whole[d]);
-            sum_sq += x * x;
-        }
-        factor = 1.0f / sqrtf(wave_sum(sum_sq) / static_cast<float>(all) + eps);
+        factor = 1.0f / sqrtf(wave_sum_squares(whole, all, lane) / static_cast<float>(all) + eps);
         weight += head * dim;
     } else if (norm_mode != 0) {
         float sum_sq = 0.f;
