@@ -49,6 +49,9 @@ struct WalkArgs {
 // shares of y meet in LDS behind the chunk.  The order of every sum depends on the sizes alone, never on what else
 // the step holds.  TIME: a decay per row, the read-out in front of the update, a bonus; else one decay per head and
 // token, the read-out behind the update.
+constexpr int kWalkAhead = 8;         // numbers of each row operand of a chunk that a thread fetches ahead
+constexpr int kWalkAheadValues = 4;   // ... and values
+
 template <int NS, bool TIME>
 __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
     extern __shared__ float4 lds4[];
@@ -83,35 +86,68 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
         S[i] = (live && n < a.rows) ? mine[static_cast<size_t>(n) * a.cols] : 0.f;
     }
     const float skip = a.skip ? a.skip[head] : 0.f;
+    // A chunk's operands are fetched into registers a chunk ahead, so that their way from memory is hidden behind
+    // the walk over the chunk before.  Every load stands in straight-line code without a condition (an index past the
+    // chunk's last number reads the last one again, a row past the memory's last its last row): behind a load under a
+    // condition the compiler waits for it before it issues the next.
+    float f_in[kWalkAhead], f_out[kWalkAhead], f_dec[TIME ? kWalkAhead : 1], f_val[kWalkAheadValues];
+    float f_scl = 1.f, f_one = 0.f;
+    const int padded_rows = RG * NS;
+#define CIE_WALK_FETCH(from_token)                                                                                    \
+    {                                                                                                                 \
+        const int fetch_n = min(a.chunk, count - (from_token));                                                       \
+        _Pragma("unroll") for (int i = 0; i < kWalkAhead; ++i) {                                                      \
+            const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * padded_rows - 1);           \
+            const int t = idx / padded_rows;                                                                          \
+            const int n = min(idx - t * padded_rows, a.rows - 1);                                                     \
+            const size_t token = static_cast<size_t>(first + (from_token) + t);                                       \
+            f_in[i] = a.in[token * a.ld_in + group * a.rows + n];                                                     \
+            f_out[i] = a.out[token * a.ld_out + group * a.rows + n];                                                  \
+            if (TIME) f_dec[i] = a.decay[token * a.ld_decay + head * a.rows + n];                                     \
+        }                                                                                                             \
+        _Pragma("unroll") for (int i = 0; i < kWalkAheadValues; ++i) {                                                \
+            const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * a.slice - 1);               \
+            const int t = idx / a.slice;                                                                              \
+            const int c = min(col0 + idx - t * a.slice, a.cols - 1);                                                  \
+            f_val[i] = a.val[static_cast<size_t>(first + (from_token) + t) * a.ld_val + head * a.cols + c];           \
+        }                                                                                                             \
+        {                                                                                                             \
+            const size_t token = static_cast<size_t>(first + (from_token) + min(static_cast<int>(threadIdx.x), fetch_n - 1)); \
+            if (a.val_scale) f_scl = a.val_scale[token * a.ld_scale + head];                                          \
+            if (!TIME) f_one = a.decay[token * a.ld_decay + head];                                                    \
+        }                                                                                                             \
+    }
+    if (count > 0) CIE_WALK_FETCH(0)
     for (int from = 0; from < count; from += a.chunk) {
         const int n_tok = min(a.chunk, count - from);
         __syncthreads();  // (the chunk before has been summed)
-        for (int idx = threadIdx.x; idx < n_tok * RG * NS; idx += blockDim.x) {
-            const int t = idx / (RG * NS);
-            const int n = idx - t * (RG * NS);
-            const int at = t * per_token + (n / NS) * pitch + n % NS;
-            const size_t token = static_cast<size_t>(first + from + t);
-            const bool real = n < a.rows;
-            const float x = real ? a.in[token * a.ld_in + group * a.rows + n] : 0.f;
-            in_s[at] = x;
-            out_s[at] = real ? a.out[token * a.ld_out + group * a.rows + n] : 0.f;
-            if (TIME) {
-                dec_s[at] = real ? a.decay[token * a.ld_decay + head * a.rows + n] : 0.f;
-                bon_s[at] = (real && a.bonus) ? a.bonus[head * a.rows + n] * x : 0.f;
+#pragma unroll
+        for (int i = 0; i < kWalkAhead; ++i) {
+            const int idx = threadIdx.x + i * blockDim.x;
+            if (idx < n_tok * padded_rows) {
+                const int t = idx / padded_rows;
+                const int n = idx - t * padded_rows;
+                const int at = t * per_token + (n / NS) * pitch + n % NS;
+                const bool real = n < a.rows;
+                in_s[at] = real ? f_in[i] : 0.f;
+                out_s[at] = real ? f_out[i] : 0.f;
+                if (TIME) {
+                    dec_s[at] = real ? f_dec[i] : 0.f;
+                    bon_s[at] = (real && a.bonus) ? a.bonus[head * a.rows + n] * f_in[i] : 0.f;
+                }
             }
         }
-        for (int idx = threadIdx.x; idx < n_tok * a.slice; idx += blockDim.x) {
-            const int t = idx / a.slice;
-            const int c = idx - t * a.slice;
-            const size_t token = static_cast<size_t>(first + from + t);
-            val_s[idx] = col0 + c < a.cols ? a.val[token * a.ld_val + head * a.cols + col0 + c] : 0.f;
+#pragma unroll
+        for (int i = 0; i < kWalkAheadValues; ++i) {
+            const int idx = threadIdx.x + i * blockDim.x;
+            if (idx < n_tok * a.slice) val_s[idx] = col0 + idx % a.slice < a.cols ? f_val[i] : 0.f;
         }
-        for (int t = threadIdx.x; t < n_tok; t += blockDim.x) {
-            const size_t token = static_cast<size_t>(first + from + t);
-            scl_s[t] = a.val_scale ? a.val_scale[token * a.ld_scale + head] : 1.f;
-            if (!TIME) dec_s[t] = a.decay[token * a.ld_decay + head];
+        if (static_cast<int>(threadIdx.x) < n_tok) {
+            scl_s[threadIdx.x] = f_scl;
+            if (!TIME) dec_s[threadIdx.x] = f_one;
         }
         __syncthreads();
+        if (from + a.chunk < count) CIE_WALK_FETCH(from + a.chunk)
         if (rg < RG) {
             const int base = rg * pitch;
             float4 in_next[Q], out_next[Q], dec_next[TIME ? Q : 1], bon_next[TIME ? Q : 1];
@@ -198,6 +234,7 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
         if (n < a.rows) mine[static_cast<size_t>(n) * a.cols] = S[i];
     }
 }
+#undef CIE_WALK_FETCH
 
 // ---------------------------------------------------------------------------------------------- the walk in blocks
 // The first form of the walk (one decay per head and token, the read-out behind the update) for sequences that
@@ -609,6 +646,12 @@ CIE_API int cie_memory_walk(void* stream, const float* decay, long ld_decay, con
                                                         static_cast<size_t>(row_groups) * slice) +
                           (time_form ? 1 : 2) * chunk4;
     if (floats * sizeof(float) > 64 * 1024) return CIE_BAD_ARGUMENT;
+    {   // what a thread fetches ahead must hold a chunk
+        const int launch = ((slice * row_groups + kWave - 1) / kWave) * kWave;
+        if (static_cast<long>(chunk) * row_groups * rows_per_thread > static_cast<long>(kWalkAhead) * launch ||
+            static_cast<long>(chunk) * slice > static_cast<long>(kWalkAheadValues) * launch || chunk > launch)
+            return CIE_BAD_ARGUMENT;
+    }
     if (sequences == 0) return CIE_OK;
     WalkArgs a{decay, ld_decay, in, ld_in, out, ld_out, heads_per_group, bonus, val, ld_val, val_scale, ld_scale,
                skip, state, seq_slot, q_start_loc, y, heads, rows, cols, slice, row_groups, chunk};

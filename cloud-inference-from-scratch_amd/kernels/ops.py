@@ -1156,6 +1156,10 @@ def plan_memory_walk(rows: int, cols: int, time_form: bool, units: int = 1) -> t
     per_token = groups * (per_thread + 4)
     floats = (4 if time_form else 2) * per_token + slice_cols + groups * slice_cols
     chunk = max(1, min(16, (WALK_LDS_BYTES - 64) // (4 * floats)))
+    # (a thread fetches the next chunk's operands into registers while it walks this one: 8 numbers of each row
+    # operand and 4 values a thread)
+    threads = -(-slice_cols * groups // 64) * 64
+    chunk = max(1, min(chunk, 8 * threads // (groups * per_thread), 4 * threads // slice_cols))
     return per_thread, groups, slice_cols, chunk
 
 
