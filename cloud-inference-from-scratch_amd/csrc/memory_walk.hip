@@ -93,23 +93,35 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
     float f_in[kWalkAhead], f_out[kWalkAhead], f_dec[TIME ? kWalkAhead : 1], f_val[kWalkAheadValues];
     float f_scl = 1.f, f_one = 0.f;
     const int padded_rows = RG * NS;
+    // which token of a chunk and which row each of the thread's numbers is, and its place in LDS: the same in every chunk
+    int slot_t[kWalkAhead], slot_n[kWalkAhead], slot_at[kWalkAhead], value_t[kWalkAheadValues], value_c[kWalkAheadValues];
+#pragma unroll
+    for (int i = 0; i < kWalkAhead; ++i) {
+        const int idx = threadIdx.x + i * blockDim.x;
+        slot_t[i] = idx / padded_rows;
+        slot_n[i] = idx - slot_t[i] * padded_rows;
+        slot_at[i] = slot_t[i] * per_token + (slot_n[i] / NS) * pitch + slot_n[i] % NS;
+    }
+#pragma unroll
+    for (int i = 0; i < kWalkAheadValues; ++i) {
+        const int idx = threadIdx.x + i * blockDim.x;
+        value_t[i] = idx / a.slice;
+        value_c[i] = idx - value_t[i] * a.slice;
+    }
 #define CIE_WALK_FETCH(from_token)                                                                                    \
     {                                                                                                                 \
         const int fetch_n = min(a.chunk, count - (from_token));                                                       \
         _Pragma("unroll") for (int i = 0; i < kWalkAhead; ++i) {                                                      \
-            const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * padded_rows - 1);           \
-            const int t = idx / padded_rows;                                                                          \
-            const int n = min(idx - t * padded_rows, a.rows - 1);                                                     \
-            const size_t token = static_cast<size_t>(first + (from_token) + t);                                       \
+            const int n = min(slot_n[i], a.rows - 1);                                                                 \
+            const size_t token = static_cast<size_t>(first + (from_token) + min(slot_t[i], fetch_n - 1));             \
             f_in[i] = a.in[token * a.ld_in + group * a.rows + n];                                                     \
             f_out[i] = a.out[token * a.ld_out + group * a.rows + n];                                                  \
             if (TIME) f_dec[i] = a.decay[token * a.ld_decay + head * a.rows + n];                                     \
         }                                                                                                             \
         _Pragma("unroll") for (int i = 0; i < kWalkAheadValues; ++i) {                                                \
-            const int idx = min(static_cast<int>(threadIdx.x + i * blockDim.x), fetch_n * a.slice - 1);               \
-            const int t = idx / a.slice;                                                                              \
-            const int c = min(col0 + idx - t * a.slice, a.cols - 1);                                                  \
-            f_val[i] = a.val[static_cast<size_t>(first + (from_token) + t) * a.ld_val + head * a.cols + c];           \
+            const int c = min(col0 + value_c[i], a.cols - 1);                                                         \
+            f_val[i] = a.val[static_cast<size_t>(first + (from_token) + min(value_t[i], fetch_n - 1)) * a.ld_val +    \
+                             head * a.cols + c];                                                                      \
         }                                                                                                             \
         {                                                                                                             \
             const size_t token = static_cast<size_t>(first + (from_token) + min(static_cast<int>(threadIdx.x), fetch_n - 1)); \
@@ -123,11 +135,9 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
         __syncthreads();  // (the chunk before has been summed)
 #pragma unroll
         for (int i = 0; i < kWalkAhead; ++i) {
-            const int idx = threadIdx.x + i * blockDim.x;
-            if (idx < n_tok * padded_rows) {
-                const int t = idx / padded_rows;
-                const int n = idx - t * padded_rows;
-                const int at = t * per_token + (n / NS) * pitch + n % NS;
+            if (slot_t[i] < n_tok) {
+                const int n = slot_n[i];
+                const int at = slot_at[i];
                 const bool real = n < a.rows;
                 in_s[at] = real ? f_in[i] : 0.f;
                 out_s[at] = real ? f_out[i] : 0.f;
@@ -139,8 +149,7 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
         }
 #pragma unroll
         for (int i = 0; i < kWalkAheadValues; ++i) {
-            const int idx = threadIdx.x + i * blockDim.x;
-            if (idx < n_tok * a.slice) val_s[idx] = col0 + idx % a.slice < a.cols ? f_val[i] : 0.f;
+            if (value_t[i] < n_tok) val_s[value_t[i] * a.slice + value_c[i]] = col0 + value_c[i] < a.cols ? f_val[i] : 0.f;
         }
         if (static_cast<int>(threadIdx.x) < n_tok) {
             scl_s[threadIdx.x] = f_scl;
