@@ -52,7 +52,9 @@ struct WalkArgs {
 constexpr int kWalkAhead = 8;         // numbers of each row operand of a chunk that a thread fetches ahead
 constexpr int kWalkAheadValues = 4;   // ... and values
 
-template <int NS, bool TIME>
+// AHEAD: the next chunk's operands are fetched into registers while this chunk is walked (sequences that bring many
+// tokens); without it a chunk is staged straight from memory (steps of single tokens, where fetching ahead only costs).
+template <int NS, bool TIME, bool AHEAD>
 __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
     extern __shared__ float4 lds4[];
     float* lds = reinterpret_cast<float*>(lds4);
@@ -96,14 +98,14 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
     // which token of a chunk and which row each of the thread's numbers is, and its place in LDS: the same in every chunk
     int slot_t[kWalkAhead], slot_n[kWalkAhead], slot_at[kWalkAhead], value_t[kWalkAheadValues], value_c[kWalkAheadValues];
 #pragma unroll
-    for (int i = 0; i < kWalkAhead; ++i) {
+    for (int i = 0; AHEAD && i < kWalkAhead; ++i) {
         const int idx = threadIdx.x + i * blockDim.x;
         slot_t[i] = idx / padded_rows;
         slot_n[i] = idx - slot_t[i] * padded_rows;
         slot_at[i] = slot_t[i] * per_token + (slot_n[i] / NS) * pitch + slot_n[i] % NS;
     }
 #pragma unroll
-    for (int i = 0; i < kWalkAheadValues; ++i) {
+    for (int i = 0; AHEAD && i < kWalkAheadValues; ++i) {
         const int idx = threadIdx.x + i * blockDim.x;
         value_t[i] = idx / a.slice;
         value_c[i] = idx - value_t[i] * a.slice;
@@ -129,12 +131,39 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
             if (!TIME) f_one = a.decay[token * a.ld_decay + head];                                                    \
         }                                                                                                             \
     }
-    if (count > 0) CIE_WALK_FETCH(0)
+    if (AHEAD && count > 0) CIE_WALK_FETCH(0)
     for (int from = 0; from < count; from += a.chunk) {
         const int n_tok = min(a.chunk, count - from);
         __syncthreads();  // (the chunk before has been summed)
+        if (!AHEAD) {
+            for (int idx = threadIdx.x; idx < n_tok * padded_rows; idx += blockDim.x) {
+                const int t = idx / padded_rows;
+                const int n = idx - t * padded_rows;
+                const int at = t * per_token + (n / NS) * pitch + n % NS;
+                const size_t token = static_cast<size_t>(first + from + t);
+                const bool real = n < a.rows;
+                const float x = real ? a.in[token * a.ld_in + group * a.rows + n] : 0.f;
+                in_s[at] = x;
+                out_s[at] = real ? a.out[token * a.ld_out + group * a.rows + n] : 0.f;
+                if (TIME) {
+                    dec_s[at] = real ? a.decay[token * a.ld_decay + head * a.rows + n] : 0.f;
+                    bon_s[at] = (real && a.bonus) ? a.bonus[head * a.rows + n] * x : 0.f;
+                }
+            }
+            for (int idx = threadIdx.x; idx < n_tok * a.slice; idx += blockDim.x) {
+                const int t = idx / a.slice;
+                const int c = idx - t * a.slice;
+                const size_t token = static_cast<size_t>(first + from + t);
+                val_s[idx] = col0 + c < a.cols ? a.val[token * a.ld_val + head * a.cols + col0 + c] : 0.f;
+            }
+            for (int t = threadIdx.x; t < n_tok; t += blockDim.x) {
+                const size_t token = static_cast<size_t>(first + from + t);
+                scl_s[t] = a.val_scale ? a.val_scale[token * a.ld_scale + head] : 1.f;
+                if (!TIME) dec_s[t] = a.decay[token * a.ld_decay + head];
+            }
+        }
 #pragma unroll
-        for (int i = 0; i < kWalkAhead; ++i) {
+        for (int i = 0; AHEAD && i < kWalkAhead; ++i) {
             if (slot_t[i] < n_tok) {
                 const int n = slot_n[i];
                 const int at = slot_at[i];
@@ -148,19 +177,21 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
             }
         }
 #pragma unroll
-        for (int i = 0; i < kWalkAheadValues; ++i) {
+        for (int i = 0; AHEAD && i < kWalkAheadValues; ++i) {
             if (value_t[i] < n_tok) val_s[value_t[i] * a.slice + value_c[i]] = col0 + value_c[i] < a.cols ? f_val[i] : 0.f;
         }
-        if (static_cast<int>(threadIdx.x) < n_tok) {
+        if (AHEAD && static_cast<int>(threadIdx.x) < n_tok) {
             scl_s[threadIdx.x] = f_scl;
             if (!TIME) dec_s[threadIdx.x] = f_one;
         }
         __syncthreads();
-        if (from + a.chunk < count) CIE_WALK_FETCH(from + a.chunk)
+        if (AHEAD && from + a.chunk < count) CIE_WALK_FETCH(from + a.chunk)
         if (rg < RG) {
             const int base = rg * pitch;
             float4 in_next[Q], out_next[Q], dec_next[TIME ? Q : 1], bon_next[TIME ? Q : 1];
-            float v_next = val_s[col] * scl_s[0];
+            // (a token's value and its scale are multiplied when the token's turn comes, not behind their loads: the
+            // product there would make the wave wait for LDS at the head of every token)
+            float v_next = val_s[col], s_next = scl_s[0];
             float d_next = TIME ? 0.f : dec_s[0];
 #pragma unroll
             for (int r = 0; r < Q; ++r) {
@@ -173,7 +204,7 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
             }
             for (int t = 0; t < n_tok; ++t) {
                 float4 in_now[Q], out_now[Q], dec_now[TIME ? Q : 1], bon_now[TIME ? Q : 1];
-                const float v = v_next;
+                const float v = v_next * s_next;
                 const float d = d_next;
 #pragma unroll
                 for (int r = 0; r < Q; ++r) {
@@ -186,7 +217,8 @@ __global__ void __launch_bounds__(512) memory_walk_kernel(WalkArgs a) {
                 }
                 const int ahead = min(t + 1, n_tok - 1);  // (the last token is read twice: no condition around the reads)
                 const int at = ahead * per_token + base;
-                v_next = val_s[ahead * a.slice + col] * scl_s[ahead];
+                v_next = val_s[ahead * a.slice + col];
+                s_next = scl_s[ahead];
                 if (!TIME) d_next = dec_s[ahead];
 #pragma unroll
                 for (int r = 0; r < Q; ++r) {
@@ -636,12 +668,14 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
 // The walk (see the head of this file).  `time_form`: a decay per row ([tokens, heads * rows]), the read-out in front of
 // the update, `bonus` if given; else one decay per head and token ([tokens, heads]) and the read-out behind the update.
 // `rows_per_thread` in {4, 8, 16, 32, 64}; `row_groups * rows_per_thread >= rows`; `slice` columns a workgroup,
-// `slice * row_groups <= 512` threads; `chunk` tokens staged at once.
+// `slice * row_groups <= 512` threads; `chunk` tokens staged at once; `ahead`: the next chunk's operands are fetched
+// into registers while a chunk is walked (for sequences that bring many tokens).
 CIE_API int cie_memory_walk(void* stream, const float* decay, long ld_decay, const float* in, long ld_in,
                             const float* out, long ld_out, int heads_per_group, const float* bonus, const float* val,
                             long ld_val, const float* val_scale, long ld_scale, const float* skip, float* state,
                             const int* seq_slot, const int* q_start_loc, float* y, int sequences, int heads, int rows,
-                            int cols, int rows_per_thread, int row_groups, int slice, int chunk, int time_form) {
+                            int cols, int rows_per_thread, int row_groups, int slice, int chunk, int time_form,
+                            int ahead) {
     if (sequences < 0 || heads <= 0 || heads > 65535 || rows <= 0 || cols <= 0 || heads_per_group <= 0 ||
         heads % heads_per_group || row_groups <= 0 || slice <= 0 || chunk <= 0 ||
         static_cast<long>(rows_per_thread) * row_groups < rows || slice * row_groups > 512 || !decay || !in || !out ||
@@ -668,9 +702,11 @@ CIE_API int cie_memory_walk(void* stream, const float* decay, long ld_decay, con
     const dim3 grid(sequences, heads, slices);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const size_t lds = floats * sizeof(float);
-#define CIE_WALK(NS)                                                                       \
-    if (time_form) memory_walk_kernel<NS, true><<<grid, threads, lds, s>>>(a);              \
-    else memory_walk_kernel<NS, false><<<grid, threads, lds, s>>>(a)
+#define CIE_WALK(NS)                                                                                \
+    if (time_form && ahead) memory_walk_kernel<NS, true, true><<<grid, threads, lds, s>>>(a);           \
+    else if (time_form) memory_walk_kernel<NS, true, false><<<grid, threads, lds, s>>>(a);             \
+    else if (ahead) memory_walk_kernel<NS, false, true><<<grid, threads, lds, s>>>(a);                 \
+    else memory_walk_kernel<NS, false, false><<<grid, threads, lds, s>>>(a)
     if (rows_per_thread == 4) { CIE_WALK(4); }
     else if (rows_per_thread == 8) { CIE_WALK(8); }
     else if (rows_per_thread == 16) { CIE_WALK(16); }

@@ -1134,6 +1134,7 @@ def gated_recurrence(y_pre: torch.Tensor, x_in: torch.Tensor, u: torch.Tensor, g
 WALK_ROWS = (4, 8, 16, 32, 64)   # rows of a memory that one thread of the walk keeps in registers
 WALK_MAX_ROWS = 1024
 WALK_LDS_BYTES = 48 * 1024
+WALK_AHEAD_FROM = 4              # tokens a sequence (on average) from which the walk fetches a chunk's operands a chunk ahead
 WALK_BLOCKS_FROM = 16            # tokens a sequence (on average) from which the first form of the walk goes in blocks
 WALK_BLOCKS_MAX_BYTES = 2 << 30  # ... while the blocks' sums fit this much scratch memory
 
@@ -1235,7 +1236,7 @@ def memory_walk(decay: torch.Tensor, in_rows: torch.Tensor, out_rows: torch.Tens
         _stream(), _ptr(decay), ld(decay), _ptr(in_rows), ld(in_rows), _ptr(out_rows), ld(out_rows), _i(heads_per_group),
         _ptr(bonus), _ptr(values), ld(values), _ptr(value_scale), ld_scale, _ptr(skip), _ptr(state), _ptr(seq_slot),
         _ptr(q_start_loc), _ptr(y), _i(sequences), _i(heads), _i(rows), _i(cols), _i(per_thread), _i(row_groups),
-        _i(slice_cols), _i(chunk), _i(1 if read_first else 0)))
+        _i(slice_cols), _i(chunk), _i(1 if read_first else 0), _i(1 if tokens >= WALK_AHEAD_FROM * max(sequences, 1) else 0)))
     return y
 
 
